@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the PULP-NN int8 kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-layers] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input: the
+pointwise 1x1 convolution 28x28x128 -> 256 channels at batch 256 (scalar
+multiplier requantisation + ReLU), the configuration the headline metric is
+quoted on.  Inputs are resident in HBM before the timed region; successive steps
+rotate through enough buffer sets (> 256 MB in total) that the Infinity Cache
+cannot hold them.  The last line printed is the JSON record.
+
+Besides the headline workload the record carries, under "layers", the other
+single-layer configurations (3x3 conv at batch 256, depthwise 3x3 stride 1 and 2
+at batch 256, the 64-bit batch-norm 3x3 conv at batch 64), each with its own
+achieved fraction of the int8 MFMA peak and of the HBM bandwidth.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA, op/s
+PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards by batch "
+                 "with no exchange, see DESIGN.md")
+
+    import numpy as np
+    import torch
+
+    from pulp_nn_amd import PulpNN, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    libs = {32: PulpNN(32), 64: PulpNN(64)}
+    for L in libs.values():
+        L.use_torch_stream()
+
+    def t(a):
+        return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def time_launches(fn, steps, warmup):
+        """fn(i) queues one step on torch's current stream (the library's stream).
+        Returns (wall ms per step, device ms per step from HIP events)."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+    def rotating(nbytes):
+        """How many buffer sets make the rotation exceed the 256 MB Infinity Cache twice over."""
+        return max(2, int(np.ceil(600e6 / nbytes)))
+
+    # ---- headline: config 1 -------------------------------------------------
+    c1 = workloads.config1(batch=256)
+    L = libs[32]
+    B, H, W, Ci = c1["x"].shape
+    Co = c1["w"].shape[0]
+    nset = rotating(c1["bytes"])
+    x0 = t(c1["x"])
+    xs = [x0] + [x0.clone() for _ in range(nset - 1)]
+    outs = [torch.zeros((B, H, W, Co), dtype=torch.uint8, device="cuda") for _ in range(nset)]
+    w, bias = t(c1["w"]), t(c1["bias"])
+    L.set_batch(B)
+
+    def step_c1(i):
+        j = i % nset
+        L.pulp_nn_pointwise_HoWo_parallel(xs[j], None, bias, outs[j], w, None, None, c1["out_mult"], c1["out_shift"],
+                                          W, H, Ci, W, H, Co, 1, 1, 0, 0, 0, 0, 1, 1, c1["relu"], c1["bn"])
+
+    wall_ms, dev_ms = time_launches(step_c1, args.steps, args.warmup)
+
+    # parity of what was just computed, on a sample of the batch
+    import oracle
+    nchk = 4
+    want = oracle.pointwise(c1["x"][:nchk], c1["w"], c1["bias"], None, None, c1["out_mult"], c1["out_shift"],
+                            c1["relu"], c1["bn"], 32)
+    got = outs[(args.steps - 1) % nset][:nchk].cpu().numpy()
+    parity = bool(np.array_equal(got, want))
+
+    gops = c1["ops"] / (wall_ms * 1e-3) / 1e9
+    rec = {
+        "metric": "int8 GOPS (2xMAC) on the pointwise conv layer at batch 256; bit-exact",
+        "value": round(gops, 1),
+        "unit": "GOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 x uint8 -> int32 (MFMA), integer requantisation to uint8",
+        "data": "synthetic (seeded PCG64: activations U[0,255], weights U[-128,127])",
+        "config": {"workload": "configs[1]: pointwise 1x1 conv 28x28x128 -> 256, batch 256, "
+                               "out_mult/out_shift requantisation + ReLU (pulp_nn_pointwise_HoWo_parallel)",
+                   "batch": B, "gemm_MxNxK": [B * H * W, Co, Ci], "buffer_sets_rotated": nset},
+        "images_per_s": round(B / (wall_ms * 1e-3), 1),
+        "device_ms_per_step": round(dev_ms, 5),
+        "parity": "bit-exact vs CPU oracle on %d images" % nchk if parity else "MISMATCH vs CPU oracle",
+        "mfma_frac": round(c1["ops"] / (dev_ms * 1e-3) / PEAK_INT8_OPS, 4),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "igemm_kernel (pointwise, 128x128 tile, scalar-multiplier epilogue)",
+            "achieved": round(c1["bytes"] / (dev_ms * 1e-3) / 1e9, 1),
+            "peak": PEAK_HBM / 1e9,
+            "unit": "GB/s",
+            "frac": round(c1["bytes"] / (dev_ms * 1e-3) / PEAK_HBM, 4),
+            "algorithmic_bytes_per_launch": c1["bytes"],
+            "traffic": None,
+        },
+    }
+
+    # ---- the other single-layer configurations ------------------------------
+    layers = []
+
+    def layer_record(name, ops, nbytes, wall, dev, ok):
+        layers.append({
+            "layer": name, "ms": round(dev, 5), "wall_ms": round(wall, 5),
+            "gops": round(ops / (dev * 1e-3) / 1e9, 1),
+            "mfma_frac": round(ops / (dev * 1e-3) / PEAK_INT8_OPS, 4),
+            "hbm_gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+            "hbm_frac": round(nbytes / (dev * 1e-3) / PEAK_HBM, 4),
+            "parity": "bit-exact" if ok else "MISMATCH"})
+
+    if not args.no_layers:
+        steps, warm = max(10, args.steps // 4), max(3, args.warmup // 4)
+
+        # config 0 at batch 256: 3x3 conv, 32-bit batch-norm
+        c0 = workloads.config0(batch=256)
+        L = libs[32]
+        nset = rotating(c0["bytes"])
+        x0 = t(c0["x"])
+        xs0 = [x0] + [x0.clone() for _ in range(min(nset, 64) - 1)]
+        outs0 = [torch.zeros((256, 16, 16, 64), dtype=torch.uint8, device="cuda") for _ in range(len(xs0))]
+        w0, b0, k0, l0 = t(c0["w"]), t(c0["bias"]), t(c0["k"]), t(c0["lam"])
+        L.set_batch(256)
+
+        def step_c0(i):
+            j = i % len(xs0)
+            L.pulp_nn_conv_Ho_parallel(xs0[j], None, b0, outs0[j], w0, k0, l0, 0, c0["out_shift"], 16, 16, 32, 16, 16,
+                                       64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
+
+        wall, dev = time_launches(step_c0, steps, warm)
+        want = oracle.conv(c0["x"][:8], c0["w"], c0["bias"], c0["k"], c0["lam"], 0, c0["out_shift"], c0["pads"],
+                           c0["strides"], 1, 1, 32)
+        layer_record(c0["name"] + "_b256", c0["ops"], c0["bytes"], wall, dev,
+                     np.array_equal(outs0[0][:8].cpu().numpy(), want))
+        del xs0, outs0
+
+        # config 2: depthwise 3x3, stride 1 through pulp_nn_depthwise_3x3_s1, stride 2 through depthwise_generic
+        for stride in (1, 2):
+            c2 = workloads.config2(batch=256, stride=stride)
+            ho = c2["out_hw"][0]
+            xin = c2["x"] if stride == 2 else np.pad(c2["x"], ((0, 0), (0, 0), (1, 1), (0, 0)))
+            nset = rotating(c2["bytes"])
+            x0 = t(xin)
+            xs2 = [x0] + [x0.clone() for _ in range(nset - 1)]
+            outs2 = [torch.zeros((256, ho, ho, 128), dtype=torch.uint8, device="cuda") for _ in range(nset)]
+            w2, b2, k2, l2 = t(c2["w"]), t(c2["bias"]), t(c2["k"]), t(c2["lam"])
+
+            if stride == 1:
+                def step_c2(i):
+                    j = i % nset
+                    L.pulp_nn_depthwise_3x3_s1(xs2[j], outs2[j], 58, 56, 128, 1, 1, w2, c2["out_shift"], 0, k2, l2,
+                                               1, 1, None)
+                want = oracle.depthwise_3x3_s1(xin[:2], c2["w"], c2["k"], c2["lam"], 0, c2["out_shift"], 1, 1, 1, 1, 32)
+            else:
+                def step_c2(i):
+                    j = i % nset
+                    L.pulp_nn_depthwise_generic(xs2[j], None, b2, outs2[j], w2, None, k2, l2, 0, c2["out_shift"],
+                                                56, 56, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1, 2, 2, 1, 1)
+                want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
+                                                (1, 1, 1, 1), (2, 2), 1, 1, 32)
+            wall, dev = time_launches(step_c2, steps, warm)
+            layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev,
+                         np.array_equal(outs2[0][:2].cpu().numpy(), want))
+            del xs2, outs2
+
+        # config 4: 64-bit batch-norm 3x3 conv at batch 64 (the MFMA-bound layer)
+        c4 = workloads.config4(batch=64, relu=1)
+        L4 = libs[64]
+        x4 = t(c4["x"])
+        nset = 4
+        xs4 = [x4] + [x4.clone() for _ in range(nset - 1)]
+        outs4 = [torch.zeros((64, 63, 63, 256), dtype=torch.uint8, device="cuda") for _ in range(nset)]
+        w4, b4, k4, l4 = t(c4["w"]), t(c4["bias"]), t(c4["k"]), t(c4["lam"])
+        L4.set_batch(64)
+
+        def step_c4(i):
+            j = i % nset
+            L4.pulp_nn_conv_Ho_parallel(xs4[j], None, b4, outs4[j], w4, k4, l4, 0, c4["out_shift"], 64, 64, 256, 63, 63,
+                                        256, 3, 3, 1, 0, 1, 0, 1, 1, 1, 1)
+
+        wall, dev = time_launches(step_c4, max(5, steps // 4), 2)
+        want = oracle.conv(c4["x"][:1], c4["w"], c4["bias"], c4["k"], c4["lam"], 0, c4["out_shift"], c4["pads"],
+                           c4["strides"], 1, 1, 64, out_hw=(63, 63))
+        layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev,
+                     np.array_equal(outs4[0][:1].cpu().numpy(), want))
+        del xs4, outs4
+        rec["layers"] = layers
+
+    # ---- CPU baseline: the oracle on this machine's host cores --------------------
+    if not args.no_cpu:
+        threads = oracle.default_threads()
+        n_img = 64
+        xs_cpu = c1["x"][:n_img]
+        oracle.pointwise(xs_cpu[:threads], c1["w"], c1["bias"], None, None, c1["out_mult"], c1["out_shift"], 1, 0, 32,
+                         nthreads=threads)
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            oracle.pointwise(xs_cpu, c1["w"], c1["bias"], None, None, c1["out_mult"], c1["out_shift"], 1, 0, 32,
+                             nthreads=threads)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el > 10.0 or reps >= 50:
+                break
+        cpu_gops = (c1["ops"] / 256 * n_img * reps) / el / 1e9
+        rec["cpu_baseline"] = {
+            "value": round(cpu_gops, 2), "unit": "GOPS", "cores": threads, "kind": "port",
+            "sample": "%d x %d images of the same workload (scalar C restatement of the reference, -O3 "
+                      "-march=native, one image row per OpenMP task), %.1f s" % (reps, n_img, el),
+            "images_per_s": round(n_img * reps / el, 1)}
+
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,64 @@
+/*
+ * pulp_nn_hip.h -- entry points this library adds to the PULP-NN kernel API.
+ *
+ * The layer functions themselves keep the names and argument lists of the
+ * reference's pulp_nn_kernels.h (see include/32bit and include/64bit); they
+ * take DEVICE pointers and return as soon as the work is queued on the
+ * library's stream.  Because those functions return void and the reference has
+ * no batch dimension, no stream and no error channel, the calls below supply
+ * them.  They have no counterpart in the reference.
+ *
+ * All state set here is per host thread.
+ */
+#ifndef PULP_NN_HIP_H
+#define PULP_NN_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  PULP_NN_HIP_OK = 0,
+  PULP_NN_HIP_ERR_ARGUMENT = 1,     /* null pointer, zero dimension, shift out of range */
+  PULP_NN_HIP_ERR_UNSUPPORTED = 2,  /* geometry outside what the reference itself handles */
+  PULP_NN_HIP_ERR_RUNTIME = 3       /* a HIP call failed */
+};
+
+/* Number of images processed by every following layer call (default 1).
+ * Images are stored back to back in every activation buffer: image i of a
+ * tensor starts i * (bytes of one image) after the pointer passed to the layer
+ * function.  Weights, bias, k and lambda are shared by all images. */
+void pulp_nn_hip_set_batch(unsigned n_images);
+unsigned pulp_nn_hip_get_batch(void);
+
+/* hipStream_t (as void*) on which following layer calls are queued; NULL is
+ * the default stream. */
+void pulp_nn_hip_set_stream(void *hip_stream);
+void *pulp_nn_hip_get_stream(void);
+
+/* Wait for everything queued on the current stream.  Returns a status code. */
+int pulp_nn_hip_sync(void);
+
+/* Status of the most recent failing layer call on this thread since the last
+ * pulp_nn_hip_clear_error(), or PULP_NN_HIP_OK.  A layer call that fails
+ * validation queues no work. */
+int pulp_nn_hip_last_error(void);
+const char *pulp_nn_hip_last_error_string(void);
+void pulp_nn_hip_clear_error(void);
+
+/* 32 or 64: the width of k / lambda this build of the library expects. */
+int pulp_nn_hip_bn_bits(void);
+
+/* Layout glue between a conv / pointwise output (HWC) and a depthwise input
+ * (CHW), which the reference leaves to the application: writes, per image,
+ * ch planes of (pad_top + dim_y + pad_bottom) x dim_x bytes, the pad rows
+ * zero.  pad_top = pad_bottom = 1 gives the row-padded plane that
+ * pulp_nn_depthwise_3x3_s1 expects. */
+void pulp_nn_hip_hwc_to_chw(const unsigned char *in_hwc, unsigned char *out_chw,
+                            unsigned dim_x, unsigned dim_y, unsigned ch,
+                            unsigned pad_top, unsigned pad_bottom);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

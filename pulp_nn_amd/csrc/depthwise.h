@@ -1,0 +1,302 @@
+// Depthwise convolution kernels: CHW input, [ch][ky][kx] weights, HWC output,
+// exactly the layouts of the reference API
+// (32bit/src/pulp_nn_depthwise_generic.c:74-81,179 and
+//  pulp_nn_depthwise_3x3_s1.c:79-85,110,145-146).
+//
+// These are bandwidth-bound VALU kernels (9 MACs per output byte), not MFMA
+// work.  One workgroup handles one image, one group of CG channels and one
+// band of RB output rows:
+//   1. stage: the (RB-1)*sy+ky input rows of every channel of the group are
+//      copied from HBM into LDS with loads that run along x and on through the
+//      following rows (the rows of a band are contiguous in a CHW plane).  Bytes
+//      are stored as a ^ 0x80 (a - 128 as int8) and everything outside the image
+//      (left / right / top / bottom padding) is stored as 0x80, so the compute
+//      phase has no border cases.  128 * sum(w) is added back per channel.
+//   2. compute: lane <-> channel.  The LDS channel stride is an odd number of
+//      dwords, so the 64 lanes of a wave read 64 different banks.  For 3x3 a
+//      lane produces 4 horizontally adjacent outputs per step from 3 (stride 1)
+//      or 4 (stride 2) dwords per input row with v_dot4_i32_i8 on byte windows,
+//      the reference's own trick (pulp_nn_depthwise_3x3_s1.c:89-91,154-159)
+//      of using the filter (K0,K1,K2,0) and its shifted copy (0,K0,K1,K2).
+//   3. store: a 4x4 byte transpose inside each lane quad (DPP + v_perm) turns
+//      "4 pixels of my channel" into "4 channels of one pixel", so that 16
+//      quads write 64 contiguous bytes of an HWC pixel.
+#pragma once
+#include "requant.h"
+
+struct DwGeom {
+  const uint8_t *in;
+  const int8_t *wt;
+  const int8_t *bias;  // may be null
+  uint8_t *out;
+  int B, CH, H, W, Ho, Wo;
+  int kx, ky, pt, pl, sx, sy;
+  int RB;       // output rows per band
+  int NR;       // staged input rows per band: (RB-1)*sy + ky
+  int LP;       // left pad columns in LDS (multiple of 4, >= pl)
+  int LWD;      // LDS row stride in dwords
+  int CSD;      // LDS channel stride in dwords (odd)
+  int bands;    // ceil(Ho / RB)
+  int cgroups;  // ceil(CH / CG)
+  int total;    // B * bands * cgroups workgroups
+  // increments of (dword, row, channel) when the staging slot index grows by 256
+  int inc_dw, inc_row, inc_c;
+  int in_align4;  // input pointer and W are multiples of 4: aligned dword loads are safe
+  int out_vec4;   // output pointer and CH are multiples of 4: dword stores are safe
+};
+
+#define DW_CG 64  // channels per workgroup (one per lane)
+
+__device__ __forceinline__ int dw_xcd_remap(int id, int total)
+{
+  const int q = total >> 3, rem = total & 7;
+  const int x = id & 7, s = id >> 3;
+  return x * q + min(x, rem) + s;
+}
+
+// Stage the input band of this workgroup into LDS (see step 1 above).
+__device__ __forceinline__ void dw_stage(const DwGeom &g, unsigned *lds, const uint8_t *img, int c0, int iy_start)
+{
+  const int tid = threadIdx.x;
+  const int slots = DW_CG * g.NR * g.LWD;
+  int dw = tid % g.LWD;
+  int t2 = tid / g.LWD;
+  int row = t2 % g.NR;
+  int c = t2 / g.NR;
+  for (int s = tid; s < slots; s += 256) {
+    unsigned v = 0;
+    const int ch = c0 + c;
+    const int iy = iy_start + row;
+    const int ix = 4 * dw - g.LP;
+    if (ch < g.CH && (unsigned)iy < (unsigned)g.H && ix + 3 >= 0 && ix < g.W) {
+      const uint8_t *src = img + ((long long)ch * g.H + iy) * g.W + ix;
+      if (g.in_align4 && ix >= 0 && ix + 3 < g.W) {
+        v = *(const unsigned *)src;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if ((unsigned)(ix + j) < (unsigned)g.W) v |= (unsigned)src[j] << (8 * j);
+      }
+    }
+    lds[c * g.CSD + row * g.LWD + dw] = v ^ 0x80808080u;
+    dw += g.inc_dw;
+    if (dw >= g.LWD) { dw -= g.LWD; row++; }
+    row += g.inc_row;
+    if (row >= g.NR) { row -= g.NR; c++; }
+    c += g.inc_c;
+  }
+}
+
+// 4x4 byte transpose across the four lanes of a quad: in: byte j of lane q =
+// element (q, j); out: byte q' of lane j' = element (q', j').
+__device__ __forceinline__ unsigned quad_transpose4x4(unsigned v, int lane)
+{
+  // exchange 16-bit halves with lane ^ 2
+  unsigned t = (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true);
+  v = (lane & 2) ? ((t >> 16) | (v & 0xFFFF0000u)) : ((v & 0x0000FFFFu) | (t << 16));
+  // exchange bytes with lane ^ 1
+  t = (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true);
+  v = (lane & 1) ? (((t >> 8) & 0x00FF00FFu) | (v & 0xFF00FF00u)) : ((v & 0x00FF00FFu) | ((t << 8) & 0xFF00FF00u));
+  return v;
+}
+
+// bytes [o, o+4) of the little-endian byte string formed by the dwords of `span`
+template <int O, int NS>
+__device__ __forceinline__ unsigned dw_window(const unsigned (&span)[NS])
+{
+  constexpr int d = O / 4, sh = O % 4;
+  if constexpr (sh == 0) return span[d];
+  else if constexpr (d + 1 < NS) return __builtin_amdgcn_alignbyte(span[d + 1], span[d], sh);
+  else return span[d] >> (8 * sh);
+}
+
+// acc += K0*byte[O] + K1*byte[O+1] + K2*byte[O+2] of the span; wA = (K0,K1,K2,0),
+// wB = (0,K0,K1,K2) saves the byte alignment when the window starts at byte 1.
+template <int O, int NS>
+__device__ __forceinline__ void dw_tap(const unsigned (&span)[NS], unsigned wA, unsigned wB, int &acc)
+{
+  if constexpr (O % 4 == 1) acc = __builtin_amdgcn_sdot4((int)span[O / 4], (int)wB, acc, false);
+  else acc = __builtin_amdgcn_sdot4((int)dw_window<O, NS>(span), (int)wA, acc, false);
+}
+
+// 3x3 depthwise, stride S (1 or 2) in both directions, left padding PL (0 or 1).
+template <int S, int PL, int MODE>
+__global__ __launch_bounds__(256) void dw3x3_kernel(DwGeom g, EpiArgs e)
+{
+  extern __shared__ unsigned dw_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  int id = dw_xcd_remap(blockIdx.x, g.total);
+  const int cg = id % g.cgroups;
+  id /= g.cgroups;
+  const int band = id % g.bands;
+  const int b = id / g.bands;
+  const int c0 = cg * DW_CG;
+  const int oy0 = band * g.RB;
+  const int rows = min(g.RB, g.Ho - oy0);
+
+  const uint8_t *img = g.in + (long long)b * g.CH * g.H * g.W;
+  dw_stage(g, dw_lds, img, c0, oy0 * S - g.pt);
+
+  // per-lane channel constants
+  const int ch = c0 + lane;
+  const bool ch_ok = ch < g.CH;
+  unsigned wA[3], wB[3];  // (K0,K1,K2,0) and (0,K0,K1,K2) per filter row
+  int corr = 0;
+  bn_t kk = 0, ll = 0;
+  if (ch_ok) {
+    int wsum = 0;
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      const int8_t *p = g.wt + (long long)ch * 9 + 3 * i;
+      const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
+      wA[i] = k0 | (k1 << 8) | (k2 << 16);
+      wB[i] = wA[i] << 8;
+      wsum += (int)p[0] + (int)p[1] + (int)p[2];
+    }
+    corr = 128 * wsum + (g.bias ? (int)g.bias[ch] : 0);
+    if (MODE == EPI_BN) {
+      kk = e.k[ch];
+      ll = e.lambda[ch];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; i++) wA[i] = wB[i] = 0;
+  }
+  __syncthreads();
+
+  // dwords per input row needed for 4 outputs: window j starts at byte
+  // (4 - PL) + S*j of the span that begins one dword left of output column 4*xg*S
+  constexpr int O0 = 4 - PL;
+  constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
+  const int xgroups = (g.Wo + 3) >> 2;
+  const int items = rows * xgroups;
+  const unsigned *lbase = dw_lds + lane * g.CSD + (g.LP >> 2) - 1;
+  uint8_t *obase = g.out + (((long long)b * g.Ho + oy0) * g.Wo) * g.CH + c0;
+
+  for (int it = wave; it < items; it += 4) {
+    const int r = it / xgroups, xg = it - r * xgroups;
+    int acc[4] = {corr, corr, corr, corr};
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      const unsigned *p = lbase + (r * S + i) * g.LWD + xg * S;
+      unsigned span[NS];
+#pragma unroll
+      for (int d = 0; d < NS; d++) span[d] = p[d];
+      dw_tap<O0, NS>(span, wA[i], wB[i], acc[0]);
+      dw_tap<O0 + S, NS>(span, wA[i], wB[i], acc[1]);
+      dw_tap<O0 + 2 * S, NS>(span, wA[i], wB[i], acc[2]);
+      dw_tap<O0 + 3 * S, NS>(span, wA[i], wB[i], acc[3]);
+    }
+    unsigned packed = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      packed |= (unsigned)requant<MODE>(acc[j], kk, ll, e.mult, e.shift) << (8 * j);
+    // lane now holds 4 pixels of its channel; after the transpose it holds 4
+    // channels (those of its quad) of pixel 4*xg + (lane & 3)
+    packed = quad_transpose4x4(packed, lane);
+    const int ox = 4 * xg + (lane & 3);
+    const int cq = lane & ~3;
+    if (ox < g.Wo) {
+      uint8_t *o = obase + ((long long)r * g.Wo + ox) * g.CH + cq;
+      if (g.out_vec4 && c0 + cq + 3 < g.CH) {
+        *(unsigned *)o = packed;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          if (c0 + cq + c < g.CH) o[c] = (uint8_t)(packed >> (8 * c));
+      }
+    }
+  }
+}
+
+// Any kernel size / stride / padding: one output per lane per step, one LDS
+// byte read per tap.  Weights are read through L1 (lane stride ky*kx bytes).
+template <int MODE>
+__global__ __launch_bounds__(256) void dw_generic_kernel(DwGeom g, EpiArgs e)
+{
+  extern __shared__ unsigned dw_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  int id = dw_xcd_remap(blockIdx.x, g.total);
+  const int cg = id % g.cgroups;
+  id /= g.cgroups;
+  const int band = id % g.bands;
+  const int b = id / g.bands;
+  const int c0 = cg * DW_CG;
+  const int oy0 = band * g.RB;
+  const int rows = min(g.RB, g.Ho - oy0);
+
+  const uint8_t *img = g.in + (long long)b * g.CH * g.H * g.W;
+  dw_stage(g, dw_lds, img, c0, oy0 * g.sy - g.pt);
+
+  const int ch = c0 + lane;
+  const bool ch_ok = ch < g.CH;
+  const int taps = g.kx * g.ky;
+  const int8_t *wp = g.wt + (long long)(ch_ok ? ch : 0) * taps;
+  int corr = 0;
+  bn_t kk = 0, ll = 0;
+  if (ch_ok) {
+    int wsum = 0;
+    for (int t = 0; t < taps; t++) wsum += (int)wp[t];
+    corr = 128 * wsum + (g.bias ? (int)g.bias[ch] : 0);
+    if (MODE == EPI_BN) {
+      kk = e.k[ch];
+      ll = e.lambda[ch];
+    }
+  }
+  __syncthreads();
+
+  const int8_t *lb = (const int8_t *)(dw_lds + lane * g.CSD) + (g.LP - g.pl);
+  const int rowbytes = g.LWD * 4;
+  uint8_t *obase = g.out + (((long long)b * g.Ho + oy0) * g.Wo) * g.CH + ch;
+  const int items = rows * g.Wo;
+  for (int it = wave; it < items; it += 4) {
+    const int r = it / g.Wo, ox = it - r * g.Wo;
+    int acc = corr;
+    const int8_t *p = lb + (r * g.sy) * rowbytes + ox * g.sx;
+    for (int fy = 0; fy < g.ky; fy++)
+      for (int fx = 0; fx < g.kx; fx++)
+        acc += (int)p[fy * rowbytes + fx] * (int)wp[fy * g.kx + fx];
+    if (ch_ok) obase[((long long)r * g.Wo + ox) * g.CH] = (uint8_t)requant<MODE>(acc, kk, ll, e.mult, e.shift);
+  }
+}
+
+// HWC -> CHW layout change with optional zero rows above and below each plane:
+// the glue between a conv / pointwise output and a depthwise input (the
+// reference leaves this step to the application).  out is [C][pad_t+H+pad_b][W].
+__global__ __launch_bounds__(256) void hwc_to_chw_kernel(const uint8_t *in, uint8_t *out, int H, int W, int C,
+                                                         int pad_t, int pad_b, int tiles_p, int tiles_c)
+{
+  // tile: 64 pixels x 64 channels through LDS
+  __shared__ uint8_t tile[64][65];
+  int id = blockIdx.x;
+  const int tc = id % tiles_c;
+  id /= tiles_c;
+  const int tp = id % tiles_p;
+  const int b = id / tiles_p;
+  const int HW = H * W;
+  const int Hp = pad_t + H + pad_b;
+  const uint8_t *src = in + (long long)b * HW * C;
+  uint8_t *dst = out + (long long)b * C * Hp * W;
+  const int p0 = tp * 64, c0 = tc * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int p = p0 + i, c = c0 + tx;
+    tile[i][tx] = (p < HW && c < C) ? src[(long long)p * C + c] : 0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, p = p0 + tx;
+    if (c < C && p < HW) dst[((long long)c * Hp + pad_t) * W + p] = tile[tx][i];
+  }
+  // zero rows
+  if (tp == 0 && (pad_t | pad_b)) {
+    for (int i = ty; i < 64; i += 4) {
+      const int c = c0 + i;
+      if (c >= C) continue;
+      for (int x = tx; x < pad_t * W; x += 64) dst[(long long)c * Hp * W + x] = 0;
+      for (int x = tx; x < pad_b * W; x += 64) dst[((long long)c * Hp + pad_t + H) * W + x] = 0;
+    }
+  }
+}

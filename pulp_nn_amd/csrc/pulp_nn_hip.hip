@@ -1,0 +1,501 @@
+// C-ABI host layer: the PULP-NN layer functions on MI355X.
+//
+// Built twice: -DPULPNN_BN_BITS=32 -> libpulpnn_hip32.so, =64 -> libpulpnn_hip64.so,
+// mirroring the reference's 32bit/ and 64bit/ trees (same symbol names, k / lambda
+// typed int32_t or int64_t).  Each function validates its arguments, picks a
+// kernel variant and queues it; nothing is allocated and no state is kept
+// besides the per-thread batch count, stream and last error.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#if PULPNN_BN_BITS == 64
+#include "../../include/64bit/pulp_nn_kernels.h"
+#else
+#include "../../include/32bit/pulp_nn_kernels.h"
+#endif
+
+#include "depthwise.h"
+#include "igemm.h"
+#include "pool.h"
+#include "requant.h"
+
+namespace {
+
+thread_local unsigned g_batch = 1;
+thread_local hipStream_t g_stream = nullptr;
+thread_local int g_err = PULP_NN_HIP_OK;
+thread_local char g_errmsg[256] = "";
+
+void set_error(int code, const char *fn, const char *msg)
+{
+  g_err = code;
+  snprintf(g_errmsg, sizeof g_errmsg, "%s: %s", fn, msg);
+}
+
+#define REQUIRE(cond, code, msg)        \
+  do {                                  \
+    if (!(cond)) {                      \
+      set_error((code), __func__, msg); \
+      return;                           \
+    }                                   \
+  } while (0)
+
+void check_launch(const char *fn)
+{
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) set_error(PULP_NN_HIP_ERR_RUNTIME, fn, hipGetErrorString(e));
+}
+
+inline bool aligned(const void *p, unsigned a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// Shift as the reference's quantisers see it, plus range validation.
+// Returns false if the shift would be undefined behaviour in the reference.
+bool epi_args(int mode, const bn_t *k, const bn_t *lambda, uint16_t out_mult, int out_shift_param, EpiArgs *e)
+{
+  e->k = k;
+  e->lambda = lambda;
+  e->mult = (int)(int16_t)out_mult;
+  if (mode == EPI_RAW) {
+    e->shift = out_shift_param;  // used as written: sum >> out_shift
+    return e->shift >= 0 && e->shift < 32;
+  }
+  e->shift = (int)(int8_t)out_shift_param;  // the quantiser functions take int8_t
+  const int lim = (mode == EPI_BN) ? PULPNN_BN_BITS : 32;
+  if (mode == EPI_BN && (!k || !lambda)) return false;
+  return e->shift >= 0 && e->shift < lim;
+}
+
+// ---- implicit GEMM dispatch -------------------------------------------------
+
+template <int TN, int WM_, int WN_, int GATHER>
+void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  constexpr int BM = 64 * WM_, BN = 16 * TN * WN_;
+  const int tiles_m = (g.M + BM - 1) / BM;
+  g.tiles_n = (g.N + BN - 1) / BN;
+  g.tiles_total = tiles_m * g.tiles_n;
+  g.vec_store = (g.N % (4 * TN) == 0) && aligned(g.out, 4 * TN);
+  dim3 grid(g.tiles_total), block(256);
+  switch (mode) {
+    case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN>), grid, block, 0, s, g, e); break;
+    case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT>), grid, block, 0, s, g, e); break;
+    case EPI_RAW: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_RAW>), grid, block, 0, s, g, e); break;
+    default: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_OUT32>), grid, block, 0, s, g, e); break;
+  }
+}
+
+template <int GATHER>
+void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  if (g.N > 64) launch_igemm_mode<4, 2, 2, GATHER>(mode, g, e, s);       // 128 px x 128 ch
+  else if (g.N > 32) launch_igemm_mode<4, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 64 ch
+  else if (g.N > 16) launch_igemm_mode<2, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 32 ch
+  else launch_igemm_mode<1, 4, 1, GATHER>(mode, g, e, s);                // 256 px x 16 ch
+}
+
+void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  const bool chunk16 = (g.Ci % 16 == 0) && aligned(g.in, 16) && aligned(g.w, 16);
+  if (chunk16) launch_igemm_tile<GATHER_CHUNK16>(mode, g, e, s);
+  else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
+}
+
+// Shared body of the six convolution entry points.
+void conv_common(const char *fn, bool pointwise, const uint8_t *in, const int8_t *bias, uint8_t *out,
+                 const int8_t *w, bn_t *k, bn_t *lambda, uint16_t out_mult, uint16_t out_shift,
+                 uint16_t dim_in_x, uint16_t dim_in_y, uint16_t ch_in, uint16_t dim_out_x, uint16_t dim_out_y,
+                 uint16_t ch_out, uint16_t kx, uint16_t ky, uint16_t pt, uint16_t pl, uint16_t sx, uint16_t sy,
+                 int flag_relu, int flag_batch_norm)
+{
+  if (!in || !out || !w) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null activation or weight pointer");
+  if (!dim_in_x || !dim_in_y || !ch_in || !dim_out_x || !dim_out_y || !ch_out)
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
+  if (pointwise) {
+    // pulp_nn_pointwise_HoWo_parallel.c:103 reads pixel (y, x) of the input for output (y, x)
+    kx = ky = 1;
+    pt = pl = 0;
+    sx = sy = 1;
+    if (dim_out_x > dim_in_x || dim_out_y > dim_in_y)
+      return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "pointwise output larger than input");
+  } else if (!kx || !ky || !sx || !sy) {
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero kernel size or stride");
+  }
+  const int mode = epi_mode(flag_relu, flag_batch_norm);
+  EpiArgs e;
+  if (!epi_args(mode, k, lambda, out_mult, out_shift, &e))
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "out_shift out of range or null k/lambda");
+  const long long M = (long long)g_batch * dim_out_x * dim_out_y;
+  if (M > 0x7fffffffLL) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+  ConvGeom g;
+  g.in = in;
+  g.w = w;
+  g.bias = bias;
+  g.out = out;
+  g.M = (int)M;
+  g.N = ch_out;
+  g.K = (int)kx * ky * ch_in;
+  g.H = dim_in_y;
+  g.W = dim_in_x;
+  g.Ci = ch_in;
+  g.Ho = dim_out_y;
+  g.Wo = dim_out_x;
+  g.HoWo = (int)dim_out_x * dim_out_y;
+  g.kx = kx;
+  g.ky = ky;
+  g.pt = pt;
+  g.pl = pl;
+  g.sx = sx;
+  g.sy = sy;
+  g.in_img = (long long)dim_in_x * dim_in_y * ch_in;
+  launch_igemm(mode, g, e, g_stream);
+  check_launch(fn);
+}
+
+void linear_common(const char *fn, int mode, const uint8_t *in, const int8_t *bias, void *out, const int8_t *w,
+                   const EpiArgs &e, uint16_t dim_vec, uint16_t num_o_neurons, int rows)
+{
+  if (!in || !out || !w) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null pointer");
+  if (!dim_vec || !num_o_neurons) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
+  ConvGeom g;
+  g.in = in;
+  g.w = w;
+  g.bias = bias;
+  g.out = out;
+  g.M = rows;
+  g.N = num_o_neurons;
+  g.K = dim_vec;
+  g.H = g.W = 1;
+  g.Ci = dim_vec;
+  g.Ho = g.Wo = g.HoWo = 1;
+  g.kx = g.ky = 1;
+  g.pt = g.pl = 0;
+  g.sx = g.sy = 1;
+  g.in_img = dim_vec;
+  launch_igemm(mode, g, e, g_stream);
+  check_launch(fn);
+}
+
+// ---- depthwise dispatch -------------------------------------------------------
+
+void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uint8_t *out, const int8_t *wt,
+                      bn_t *k, bn_t *lambda, uint16_t out_mult, int out_shift, int W, int H, int Wo, int Ho, int CH,
+                      int kx, int ky, int pt, int pl, int sx, int sy, int mode)
+{
+  if (!in || !out || !wt) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null activation or weight pointer");
+  if (W <= 0 || H <= 0 || Wo <= 0 || Ho <= 0 || CH <= 0 || kx <= 0 || ky <= 0 || sx <= 0 || sy <= 0)
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
+  EpiArgs e;
+  if (!epi_args(mode, k, lambda, out_mult, out_shift, &e))
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "out_shift out of range or null k/lambda");
+  // the accumulators of these kernels fit easily; guard the i32 sum anyway
+  if ((long long)kx * ky > 4096) return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "kernel too large");
+
+  DwGeom g;
+  g.in = in;
+  g.wt = wt;
+  g.bias = bias;
+  g.out = out;
+  g.B = (int)g_batch;
+  g.CH = CH;
+  g.H = H;
+  g.W = W;
+  g.Ho = Ho;
+  g.Wo = Wo;
+  g.kx = kx;
+  g.ky = ky;
+  g.pt = pt;
+  g.pl = pl;
+  g.sx = sx;
+  g.sy = sy;
+  const bool fast = kx == 3 && ky == 3 && sx == sy && (sx == 1 || sx == 2) && (pl == 0 || pl == 1);
+  g.LP = pl > 4 ? ((pl + 3) & ~3) : 4;
+  int need_bytes;  // bytes of an LDS row the compute phase may touch
+  if (fast) {
+    const int xgroups = (Wo + 3) / 4;
+    const int ns = ((4 - pl) + 3 * sx + 2) / 4 + 1;
+    need_bytes = 4 * (g.LP / 4 - 1 + (xgroups - 1) * sx + ns);
+  } else {
+    need_bytes = g.LP - pl + (Wo - 1) * sx + kx;
+  }
+  const int img_bytes = g.LP + W + 1;
+  g.LWD = ((need_bytes > img_bytes ? need_bytes : img_bytes) + 3) / 4;
+  const int max_csd = 255;  // 64 channels x 255 dwords = 63.75 KiB of LDS
+  int nr_max = max_csd / g.LWD;
+  if (nr_max < ky) return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "image too wide for the LDS tile");
+  int rb_max = (nr_max - ky) / sy + 1;
+  if (rb_max > Ho) rb_max = Ho;
+  g.bands = (Ho + rb_max - 1) / rb_max;
+  g.RB = (Ho + g.bands - 1) / g.bands;
+  g.bands = (Ho + g.RB - 1) / g.RB;
+  g.NR = (g.RB - 1) * sy + ky;
+  g.CSD = (g.NR * g.LWD) | 1;
+  g.cgroups = (CH + DW_CG - 1) / DW_CG;
+  const long long total = (long long)g.B * g.bands * g.cgroups;
+  if (total > 0x7fffffffLL) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+  g.total = (int)total;
+  g.inc_dw = 256 % g.LWD;
+  const int carry = 256 / g.LWD;
+  g.inc_row = carry % g.NR;
+  g.inc_c = carry / g.NR;
+  g.in_align4 = aligned(in, 4) && (W % 4 == 0);
+  g.out_vec4 = aligned(out, 4) && (CH % 4 == 0);
+  const size_t lds = (size_t)DW_CG * g.CSD * 4;
+  dim3 grid(g.total), block(256);
+#define DW_LAUNCH(KERNEL)                                                                   \
+  switch (mode) {                                                                           \
+    case EPI_BN: hipLaunchKernelGGL((KERNEL<EPI_BN>), grid, block, lds, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((KERNEL<EPI_MULT>), grid, block, lds, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((KERNEL<EPI_RAW>), grid, block, lds, g_stream, g, e); break;        \
+  }
+#define DW3(S, PL, M) dw3x3_kernel<S, PL, M>
+  if (fast) {
+    if (sx == 1 && pl == 1) { switch (mode) {
+      case EPI_BN: hipLaunchKernelGGL((DW3(1, 1, EPI_BN)), grid, block, lds, g_stream, g, e); break;
+      case EPI_MULT: hipLaunchKernelGGL((DW3(1, 1, EPI_MULT)), grid, block, lds, g_stream, g, e); break;
+      default: hipLaunchKernelGGL((DW3(1, 1, EPI_RAW)), grid, block, lds, g_stream, g, e); break; }
+    } else if (sx == 1) { switch (mode) {
+      case EPI_BN: hipLaunchKernelGGL((DW3(1, 0, EPI_BN)), grid, block, lds, g_stream, g, e); break;
+      case EPI_MULT: hipLaunchKernelGGL((DW3(1, 0, EPI_MULT)), grid, block, lds, g_stream, g, e); break;
+      default: hipLaunchKernelGGL((DW3(1, 0, EPI_RAW)), grid, block, lds, g_stream, g, e); break; }
+    } else if (pl == 1) { switch (mode) {
+      case EPI_BN: hipLaunchKernelGGL((DW3(2, 1, EPI_BN)), grid, block, lds, g_stream, g, e); break;
+      case EPI_MULT: hipLaunchKernelGGL((DW3(2, 1, EPI_MULT)), grid, block, lds, g_stream, g, e); break;
+      default: hipLaunchKernelGGL((DW3(2, 1, EPI_RAW)), grid, block, lds, g_stream, g, e); break; }
+    } else { switch (mode) {
+      case EPI_BN: hipLaunchKernelGGL((DW3(2, 0, EPI_BN)), grid, block, lds, g_stream, g, e); break;
+      case EPI_MULT: hipLaunchKernelGGL((DW3(2, 0, EPI_MULT)), grid, block, lds, g_stream, g, e); break;
+      default: hipLaunchKernelGGL((DW3(2, 0, EPI_RAW)), grid, block, lds, g_stream, g, e); break; }
+    }
+  } else {
+    DW_LAUNCH(dw_generic_kernel)
+  }
+#undef DW3
+#undef DW_LAUNCH
+  check_launch(fn);
+}
+
+bool pool_geom(const char *fn, PoolGeom *g, uint8_t *in, uint8_t *out, uint16_t W, uint16_t H, uint16_t C,
+               uint16_t Wo, uint16_t Ho, uint16_t kx, uint16_t ky, uint16_t pt, uint16_t pb, uint16_t pl,
+               uint16_t pr, uint16_t sx, uint16_t sy)
+{
+  if (!in || !out) { set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null pointer"); return false; }
+  if (!W || !H || !C || !Wo || !Ho || !kx || !ky || !sx || !sy) {
+    set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
+    return false;
+  }
+  g->in = in;
+  g->out = out;
+  g->B = (int)g_batch;
+  g->H = H;
+  g->W = W;
+  g->C = C;
+  g->Ho = Ho;
+  g->Wo = Wo;
+  g->kx = kx;
+  g->ky = ky;
+  g->sx = sx;
+  g->sy = sy;
+  g->pt = pt;
+  g->pb = pb;
+  g->pl = pl;
+  g->pr = pr;
+  g->cgroups = (C + 3) / 4;
+  g->vec4 = (C % 4 == 0) && aligned(in, 4) && aligned(out, 4);
+  g->total = (long long)g->B * Ho * Wo * g->cgroups;
+  if ((g->total + 255) / 256 > 0x7fffffffLL) {
+    set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+    return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+// ---- added entry points -----------------------------------------------------------
+
+extern "C" {
+
+void pulp_nn_hip_set_batch(unsigned n_images) { g_batch = n_images ? n_images : 1; }
+unsigned pulp_nn_hip_get_batch(void) { return g_batch; }
+void pulp_nn_hip_set_stream(void *hip_stream) { g_stream = (hipStream_t)hip_stream; }
+void *pulp_nn_hip_get_stream(void) { return (void *)g_stream; }
+
+int pulp_nn_hip_sync(void)
+{
+  hipError_t e = hipStreamSynchronize(g_stream);
+  if (e != hipSuccess) {
+    set_error(PULP_NN_HIP_ERR_RUNTIME, __func__, hipGetErrorString(e));
+    return PULP_NN_HIP_ERR_RUNTIME;
+  }
+  return PULP_NN_HIP_OK;
+}
+
+int pulp_nn_hip_last_error(void) { return g_err; }
+const char *pulp_nn_hip_last_error_string(void) { return g_errmsg; }
+void pulp_nn_hip_clear_error(void)
+{
+  g_err = PULP_NN_HIP_OK;
+  g_errmsg[0] = 0;
+}
+int pulp_nn_hip_bn_bits(void) { return PULPNN_BN_BITS; }
+
+void pulp_nn_hip_hwc_to_chw(const unsigned char *in_hwc, unsigned char *out_chw, unsigned dim_x, unsigned dim_y,
+                            unsigned ch, unsigned pad_top, unsigned pad_bottom)
+{
+  REQUIRE(in_hwc && out_chw, PULP_NN_HIP_ERR_ARGUMENT, "null pointer");
+  REQUIRE(dim_x && dim_y && ch, PULP_NN_HIP_ERR_ARGUMENT, "zero dimension");
+  const int tiles_p = (int)((dim_x * dim_y + 63) / 64), tiles_c = (int)((ch + 63) / 64);
+  const long long total = (long long)g_batch * tiles_p * tiles_c;
+  REQUIRE(total <= 0x7fffffffLL, PULP_NN_HIP_ERR_ARGUMENT, "batch too large");
+  hipLaunchKernelGGL(hwc_to_chw_kernel, dim3((unsigned)total), dim3(256), 0, g_stream, in_hwc, out_chw, (int)dim_y,
+                     (int)dim_x, (int)ch, (int)pad_top, (int)pad_bottom, tiles_p, tiles_c);
+  check_launch(__func__);
+}
+
+// ---- the reference API ------------------------------------------------------------
+
+#define CONV_FORWARD(NAME, POINTWISE)                                                                   \
+  void NAME(PULP_NN_CONV_ARGS)                                                                          \
+  {                                                                                                     \
+    (void)pIm2ColBuffer;                                                                                \
+    (void)padding_y_bottom;                                                                             \
+    (void)padding_x_right;                                                                              \
+    conv_common(#NAME, POINTWISE, pInBuffer, bias, pOutBuffer, pWeight, k, lambda, out_mult, out_shift, \
+                dim_in_x, dim_in_y, ch_in, dim_out_x, dim_out_y, ch_out, dim_kernel_x, dim_kernel_y,    \
+                padding_y_top, padding_x_left, stride_x, stride_y, flag_relu, flag_batch_norm);         \
+  }
+
+CONV_FORWARD(pulp_nn_conv_Ho_parallel, false)
+CONV_FORWARD(pulp_nn_conv_Co_parallel, false)
+CONV_FORWARD(pulp_nn_conv_HoWo_parallel, false)
+CONV_FORWARD(pulp_nn_pointwise_HoWo_parallel, true)
+CONV_FORWARD(pulp_nn_pointwise_Ho_parallel, true)
+CONV_FORWARD(pulp_nn_pointwise_Co_parallel, true)
+
+void pulp_nn_linear(uint8_t *pInBuffer, int8_t *bias, uint8_t *pOutBuffer, int8_t *pWeights, bn_t *k, bn_t *lambda,
+                    uint16_t out_mult, int8_t out_shift, uint16_t dim_vec, uint16_t num_o_neurons, int flag_relu,
+                    int flag_batch_norm)
+{
+  const int mode = epi_mode(flag_relu, flag_batch_norm);
+  EpiArgs e;
+  REQUIRE(epi_args(mode, k, lambda, out_mult, out_shift, &e), PULP_NN_HIP_ERR_ARGUMENT,
+          "out_shift out of range or null k/lambda");
+  linear_common(__func__, mode, pInBuffer, bias, pOutBuffer, pWeights, e, dim_vec, num_o_neurons, (int)g_batch);
+}
+
+void pulp_nn_linear_out_32(uint8_t *pInBuffer, int8_t *bias, int32_t *pOutBuffer, int8_t *pWeights, uint16_t dim_vec,
+                           uint16_t num_o_neurons)
+{
+  REQUIRE(!bias || aligned(bias, 4), PULP_NN_HIP_ERR_ARGUMENT, "bias must be 4-byte aligned (it holds int32 values)");
+  REQUIRE(aligned(pOutBuffer, 4), PULP_NN_HIP_ERR_ARGUMENT, "output must be 4-byte aligned");
+  EpiArgs e = {nullptr, nullptr, 0, 0};
+  linear_common(__func__, EPI_OUT32, pInBuffer, bias, pOutBuffer, pWeights, e, dim_vec, num_o_neurons, (int)g_batch);
+}
+
+uint8_t *pulp_nn_matmul(const int8_t *pWeight, uint8_t *pInBuffer, uint16_t ch_out, uint16_t num_col_im2col,
+                        uint16_t out_shift, uint16_t out_mult, bn_t *k, bn_t *lambda, const int8_t *bias, uint8_t *pOut,
+                        uint8_t *pOut2, int flag_relu, int flag_batch_norm)
+{
+  const int mode = epi_mode(flag_relu, flag_batch_norm);
+  EpiArgs e;
+  if (!epi_args(mode, k, lambda, out_mult, out_shift, &e)) {
+    set_error(PULP_NN_HIP_ERR_ARGUMENT, __func__, "out_shift out of range or null k/lambda");
+    return pOut;
+  }
+  if (!pOut || !pOut2) {
+    set_error(PULP_NN_HIP_ERR_ARGUMENT, __func__, "null pointer");
+    return pOut;
+  }
+  if (pOut2 == pOut + ch_out) {
+    linear_common(__func__, mode, pInBuffer, bias, pOut, pWeight, e, num_col_im2col, ch_out, 2);
+  } else {
+    linear_common(__func__, mode, pInBuffer, bias, pOut, pWeight, e, num_col_im2col, ch_out, 1);
+    linear_common(__func__, mode, pInBuffer + num_col_im2col, bias, pOut2, pWeight, e, num_col_im2col, ch_out, 1);
+  }
+  return pOut + 2 * (size_t)ch_out;
+}
+
+void pulp_nn_maxpool(uint8_t *Im_in, uint8_t *Im_out, uint16_t dim_im_in_x, uint16_t dim_im_in_y, uint16_t ch_im_in,
+                     uint16_t dim_im_out_x, uint16_t dim_im_out_y, uint16_t dim_kernel_x, uint16_t dim_kernel_y,
+                     uint16_t padding_t, uint16_t padding_b, uint16_t padding_l, uint16_t padding_r, uint16_t stride_x,
+                     uint16_t stride_y)
+{
+  PoolGeom g;
+  if (!pool_geom(__func__, &g, Im_in, Im_out, dim_im_in_x, dim_im_in_y, ch_im_in, dim_im_out_x, dim_im_out_y,
+                 dim_kernel_x, dim_kernel_y, padding_t, padding_b, padding_l, padding_r, stride_x, stride_y))
+    return;
+  // The reference's in-place x pass re-reads columns it has already overwritten
+  // when a window starts left of the column it is stored to, i.e. for some
+  // i_x >= 1 with i_x*stride_x - padding_l < i_x (pulp_nn_maxpool.c:58-94).
+  REQUIRE(padding_l == 0 || (int)stride_x - 1 >= (int)padding_l, PULP_NN_HIP_ERR_UNSUPPORTED,
+          "left padding this large makes the reference's in-place x pass order dependent");
+  hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((g.total + 255) / 256)), dim3(256), 0, g_stream, g);
+  check_launch(__func__);
+}
+
+void pulp_nn_avgpool(uint8_t *Im_in, uint8_t *Im_out, bn_t lambda, uint16_t out_shift, bn_t out_add,
+                     uint16_t dim_im_in_x, uint16_t dim_im_in_y, uint16_t ch_im_in, uint16_t dim_im_out_x,
+                     uint16_t dim_im_out_y, uint16_t dim_kernel_x, uint16_t dim_kernel_y, uint16_t padding_t,
+                     uint16_t padding_b, uint16_t padding_l, uint16_t padding_r, uint16_t stride_x, uint16_t stride_y,
+                     int flag_requant)
+{
+  PoolGeom g;
+  if (!pool_geom(__func__, &g, Im_in, Im_out, dim_im_in_x, dim_im_in_y, ch_im_in, dim_im_out_x, dim_im_out_y,
+                 dim_kernel_x, dim_kernel_y, padding_t, padding_b, padding_l, padding_r, stride_x, stride_y))
+    return;
+  REQUIRE(!flag_requant || out_shift < PULPNN_BN_BITS, PULP_NN_HIP_ERR_ARGUMENT, "out_shift out of range");
+  REQUIRE((long long)dim_kernel_x * dim_kernel_y * 255 < 0xffffffffLL, PULP_NN_HIP_ERR_UNSUPPORTED, "window too large");
+  AvgArgs a = {(long long)lambda, (long long)out_add, (int)out_shift, flag_requant};
+  hipLaunchKernelGGL(avgpool_kernel, dim3((unsigned)((g.total + 255) / 256)), dim3(256), 0, g_stream, g, a);
+  check_launch(__func__);
+}
+
+void pulp_nn_add(uint8_t *Im_in_1, uint8_t *Im_in_2, uint8_t *Im_out, uint16_t out_mult1, uint16_t out_mult2,
+                 uint16_t out_shift, uint16_t dim_im_in_h, uint16_t dim_im_in_w, uint16_t ch_im_in)
+{
+  REQUIRE(Im_in_1 && Im_in_2 && Im_out, PULP_NN_HIP_ERR_ARGUMENT, "null pointer");
+  REQUIRE(dim_im_in_h && dim_im_in_w && ch_im_in, PULP_NN_HIP_ERR_ARGUMENT, "zero dimension");
+  const int d = (int)(int8_t)out_shift;  // pulp_nn_add_quant_u8 takes the shift as int8_t
+  REQUIRE(d >= 0 && d < 32, PULP_NN_HIP_ERR_ARGUMENT, "out_shift out of range");
+  const long long n = (long long)g_batch * dim_im_in_h * dim_im_in_w * ch_im_in;
+  const long long threads = (n + 15) / 16;
+  REQUIRE((threads + 255) / 256 <= 0x7fffffffLL, PULP_NN_HIP_ERR_ARGUMENT, "batch too large");
+  const int vec16 = aligned(Im_in_1, 16) && aligned(Im_in_2, 16) && aligned(Im_out, 16);
+  hipLaunchKernelGGL(add_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, g_stream, Im_in_1, Im_in_2,
+                     Im_out, n, (int)(int16_t)out_mult1, (int)(int16_t)out_mult2, d, vec16);
+  check_launch(__func__);
+}
+
+#define DW_FORWARD(NAME)                                                                                       \
+  void NAME(PULP_NN_DW_ARGS)                                                                                   \
+  {                                                                                                            \
+    (void)bufferC;                                                                                             \
+    (void)bufferB;                                                                                             \
+    (void)ch_im_in;                                                                                            \
+    (void)padding_y_bottom;                                                                                    \
+    (void)padding_x_right;                                                                                     \
+    depthwise_common(#NAME, Im_in, bias, Im_out, wt, k, lambda, out_mult, out_shift, dim_im_in_x, dim_im_in_y, \
+                     dim_im_out_x, dim_im_out_y, ch_im_out, dim_kernel_x, dim_kernel_y, padding_y_top,         \
+                     padding_x_left, stride_x, stride_y, epi_mode(FLAG_RELU, FLAG_BATCH_NORM, true));          \
+  }
+
+DW_FORWARD(pulp_nn_depthwise_generic)
+DW_FORWARD(pulp_nn_depthwise_generic_less_4_weights)
+
+void pulp_nn_depthwise_3x3_s1(uint8_t *In_Img, uint8_t *Out_Img, int R, int C, int CH, int p_l, int p_r,
+                              int8_t *Kernel, int8_t out_shift, uint16_t out_mult, bn_t *kappa, bn_t *lambda,
+                              int flag_relu, int flag_batch_norm, unsigned int *memory_chan)
+{
+  (void)memory_chan;
+  REQUIRE(R >= 3 && C >= 2 && CH >= 1, PULP_NN_HIP_ERR_ARGUMENT, "plane too small");
+  REQUIRE(R <= 65535 + 2 && C <= 65535 && CH <= 65535, PULP_NN_HIP_ERR_ARGUMENT, "dimension too large");
+  // Only for p_l = p_r = 1 and even C do the reference's three row pointers land on
+  // the start of the next row after each output row (pulp_nn_depthwise_3x3_s1.c:141-223).
+  REQUIRE(p_l == 1 && p_r == 1 && (C % 2) == 0, PULP_NN_HIP_ERR_UNSUPPORTED,
+          "only p_l = p_r = 1 with even C is well defined in the reference");
+  depthwise_common(__func__, In_Img, nullptr, Out_Img, Kernel, kappa, lambda, out_mult, out_shift, C, R, C, R - 2, CH,
+                   3, 3, 0, 1, 1, 1, epi_mode(flag_relu, flag_batch_norm));
+}
+
+}  // extern "C"

@@ -1,0 +1,281 @@
+"""GPU parity: every entry point of the C ABI against the CPU oracle, bit-exact.
+
+All comparisons are integer / byte work, so the bar is equality of every element."""
+import numpy as np
+import pytest
+
+import oracle
+from gpu_helpers import (add, assert_same, avgpool, conv, depthwise_3x3_s1, depthwise_generic, linear,
+                         linear_out_32, maxpool, nn, rand_s8, rand_u8, rng_for)
+
+pytestmark = pytest.mark.gpu
+
+CONV_GEOMS = [
+    # B, H, W, Ci, Co, ky, kx, pads(t,b,l,r), strides(sx,sy)
+    (2, 16, 16, 32, 64, 3, 3, (1, 1, 1, 1), (1, 1)),    # config 0 geometry
+    (3, 9, 7, 5, 6, 3, 3, (1, 1, 1, 1), (1, 1)),        # Ci, Co not multiples of anything
+    (2, 11, 13, 3, 7, 3, 3, (1, 0, 1, 0), (1, 1)),      # asymmetric padding
+    (2, 12, 12, 8, 10, 3, 3, (1, 1, 1, 1), (2, 2)),     # stride 2
+    (1, 10, 9, 6, 5, 5, 3, (2, 2, 1, 1), (1, 1)),       # ky != kx
+    (2, 16, 16, 3, 16, 3, 3, (1, 1, 1, 1), (2, 2)),     # MobileNet stem style
+    (1, 12, 10, 16, 130, 3, 3, (1, 1, 1, 1), (1, 1)),   # Co tail across two 128-wide tiles
+    (2, 9, 9, 48, 24, 3, 3, (1, 1, 1, 1), (1, 1)),      # Ci multiple of 16 but K slices straddle taps
+    (1, 7, 9, 64, 40, 1, 1, (0, 0, 0, 0), (1, 1)),      # 1x1 through the standard conv entry point
+    (1, 20, 20, 256, 32, 3, 3, (1, 0, 1, 0), (1, 1)),   # config 4 style channels, K = 2304
+]
+FLAGS = [(1, 1), (1, 0), (0, 0), (0, 1), (2, 0)]
+
+
+def bn_params(r, n, bn_bits):
+    if bn_bits == 32:
+        return r.integers(256, 1025, n), r.integers(-2 ** 16, 2 ** 16 + 1, n), 20
+    return r.integers(2 ** 20, 2 ** 24 + 1, n), r.integers(-2 ** 36, 2 ** 36 + 1, n), 38
+
+
+def pick_shift(relu, bn, bn_shift, K):
+    if relu and bn:
+        return bn_shift
+    lg = int(np.log2(max(K, 2) ** 0.5 * 128 * 74))      # typical |acc|
+    return (lg + 10 - 7) if relu == 1 else max(lg - 7, 0)
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", FLAGS)
+@pytest.mark.parametrize("geom", CONV_GEOMS, ids=lambda g: "x".join(map(str, g[:7])))
+def test_conv(geom, flags, bn_bits):
+    B, H, W, Ci, Co, ky, kx, pads, strides = geom
+    relu, bn = flags
+    r = rng_for(1000 + 17 * relu + bn + bn_bits)
+    x, w, b = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, ky, kx, Ci)), rand_s8(r, (Co,))
+    k, lam, bshift = bn_params(r, Co, bn_bits)
+    mult = int(r.integers(256, 1025))
+    shift = pick_shift(relu, bn, bshift, ky * kx * Ci)
+    want = oracle.conv(x, w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
+    got = conv(x, w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
+    assert_same(got, want, "conv")
+    assert want.max() > 0 and (want < 255).any(), "degenerate case"
+
+
+def test_conv_variants_and_null_bias():
+    B, H, W, Ci, Co = 2, 10, 12, 32, 20
+    r = rng_for(7)
+    x, w = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, 3, 3, Ci))
+    k, lam = r.integers(256, 1025, Co), r.integers(-2 ** 16, 2 ** 16, Co)
+    want = oracle.conv(x, w, None, k, lam, 0, 20, (1, 1, 1, 1), (1, 1), 1, 1)
+    for fn in ("pulp_nn_conv_Ho_parallel", "pulp_nn_conv_HoWo_parallel", "pulp_nn_conv_Co_parallel"):
+        assert_same(conv(x, w, None, k, lam, 0, 20, (1, 1, 1, 1), (1, 1), 1, 1, fn=fn), want, fn)
+
+
+PW_GEOMS = [
+    # B, H, W, Ci, Co
+    (4, 28, 28, 128, 256),   # config 1 geometry, small batch
+    (3, 7, 5, 24, 13),
+    (2, 8, 8, 16, 32),
+    (2, 4, 4, 512, 512),
+    (1, 9, 11, 3, 100),
+    (5, 3, 3, 70, 64),
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", FLAGS)
+@pytest.mark.parametrize("geom", PW_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_pointwise(geom, flags, bn_bits):
+    B, H, W, Ci, Co = geom
+    relu, bn = flags
+    r = rng_for(2000 + 17 * relu + bn + bn_bits)
+    x, w, b = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, 1, 1, Ci)), rand_s8(r, (Co,))
+    k, lam, bshift = bn_params(r, Co, bn_bits)
+    mult = int(r.integers(256, 1025))
+    shift = pick_shift(relu, bn, bshift, Ci)
+    want = oracle.pointwise(x, w, b, k, lam, mult, shift, relu, bn, bn_bits)
+    for fn in ("pulp_nn_pointwise_HoWo_parallel", "pulp_nn_pointwise_Ho_parallel", "pulp_nn_pointwise_Co_parallel"):
+        # stride / padding / kernel arguments are deliberately nonsense: the reference ignores them
+        got = conv(x, w, b, k, lam, mult, shift, (3, 3, 3, 3), (2, 2), relu, bn, bn_bits, out_hw=(H, W), fn=fn)
+        assert_same(got, want, fn)
+
+
+def test_pointwise_output_smaller_than_input():
+    r = rng_for(3)
+    x, w = rand_u8(r, (2, 6, 8, 16)), rand_s8(r, (3, 1, 1, 16))
+    want = oracle.pointwise(x, w, None, None, None, 0, 6, 0, 0, out_hw=(4, 5))
+    got = conv(x, w, None, None, None, 0, 6, (0, 0, 0, 0), (1, 1), 0, 0, out_hw=(4, 5),
+               fn="pulp_nn_pointwise_HoWo_parallel")
+    assert_same(got, want, "pointwise crop")
+
+
+DW_GEOMS = [
+    # B, CH, H, W, ky, kx, pads, strides
+    (2, 128, 56, 56, 3, 3, (1, 1, 1, 1), (2, 2)),    # config 2 stride 2
+    (2, 8, 12, 12, 3, 3, (1, 1, 1, 1), (1, 1)),
+    (2, 70, 9, 11, 3, 3, (1, 1, 1, 1), (2, 2)),      # odd sizes, channel tail
+    (1, 16, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1)),     # MobileNet block 1
+    (1, 3, 10, 8, 5, 5, (2, 2, 2, 2), (1, 1)),
+    (2, 4, 7, 9, 3, 5, (1, 1, 2, 2), (1, 1)),
+    (1, 6, 8, 8, 1, 1, (0, 0, 0, 0), (1, 1)),
+    (1, 2, 6, 6, 2, 2, (0, 0, 0, 0), (2, 2)),
+    (1, 5, 9, 9, 3, 3, (0, 0, 0, 0), (1, 1)),        # no padding: pl = 0 fast path
+    (1, 5, 11, 11, 3, 3, (0, 0, 0, 0), (2, 2)),
+    (1, 4, 10, 230, 3, 3, (1, 1, 1, 1), (1, 1)),     # wide image: few rows per band
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", [(1, 1), (1, 0), (0, 0), (2, 0)])
+@pytest.mark.parametrize("geom", DW_GEOMS, ids=lambda g: "x".join(map(str, g[:6])) + "s%d" % g[7][0])
+def test_depthwise_generic(geom, flags, bn_bits):
+    B, CH, H, W, ky, kx, pads, strides = geom
+    relu, bn = flags
+    r = rng_for(3000 + 17 * relu + bn + bn_bits)
+    x, wt, b = rand_u8(r, (B, CH, H, W)), rand_s8(r, (CH, ky, kx)), rand_s8(r, (CH,))
+    if bn_bits == 32:
+        k, lam, bshift = r.integers(2 ** 12, 2 ** 14 + 1, CH), r.integers(-2 ** 16, 2 ** 16 + 1, CH), 16
+    else:
+        k, lam, bshift = r.integers(2 ** 20, 2 ** 24 + 1, CH), r.integers(-2 ** 36, 2 ** 36 + 1, CH), 28
+    shift = bshift if (relu and bn) else (14 if relu else 6)
+    want = oracle.depthwise_generic(x, wt, b, k, lam, 900, shift, pads, strides, relu, bn, bn_bits)
+    for fn in ("pulp_nn_depthwise_generic", "pulp_nn_depthwise_generic_less_4_weights"):
+        got = depthwise_generic(x, wt, b, k, lam, 900, shift, pads, strides, relu, bn, bn_bits, fn=fn)
+        assert_same(got, want, fn)
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", [(1, 1), (1, 0), (0, 0)])
+@pytest.mark.parametrize("shape", [(2, 128, 56, 56), (2, 5, 7, 6), (1, 3, 1, 2), (3, 66, 12, 20)])
+def test_depthwise_3x3_s1(shape, flags, bn_bits):
+    B, CH, H, W = shape
+    relu, bn = flags
+    r = rng_for(4000 + relu + bn)
+    x, kern = rand_u8(r, (B, CH, H, W)), rand_s8(r, (CH, 3, 3))
+    kern[0] = 127       # same-sign taps drive the 32-bit batch-norm product past 2^31
+    k, lam = r.integers(2 ** 12, 2 ** 14 + 1, CH), r.integers(-2 ** 16, 2 ** 16 + 1, CH)
+    k[0] = 2 ** 14
+    shift = 16 if (relu and bn) else (13 if relu else 5)
+    xpad = np.pad(x, ((0, 0), (0, 0), (1, 1), (0, 0)))
+    want = oracle.depthwise_3x3_s1(xpad, kern, k, lam, 600, shift, 1, 1, relu, bn, bn_bits)
+    got = depthwise_3x3_s1(xpad, kern, k, lam, 600, shift, relu, bn, bn_bits)
+    assert_same(got, want, "depthwise_3x3_s1")
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("dims", [(64, 1024, 4096), (256, 512, 1000), (3, 37, 11), (1, 512, 1000), (5, 100, 70)])
+def test_linear(dims, bn_bits):
+    B, K, N = dims
+    r = rng_for(5000 + K)
+    x, w, b = rand_u8(r, (B, K)), rand_s8(r, (N, K)), rand_s8(r, (N,))
+    k, lam, bshift = bn_params(r, N, bn_bits)
+    for relu, bn in FLAGS:
+        shift = pick_shift(relu, bn, bshift, K)
+        want = oracle.linear(x, w, b, k, lam, 800, shift, relu, bn, bn_bits)
+        assert_same(linear(x, w, b, k, lam, 800, shift, relu, bn, bn_bits), want, "linear %d %d" % (relu, bn))
+
+
+@pytest.mark.parametrize("dims", [(256, 512, 1000), (3, 37, 11), (2, 1024, 64)])
+def test_linear_out_32(dims):
+    B, K, N = dims
+    r = rng_for(6000 + K)
+    x, w = rand_u8(r, (B, K)), rand_s8(r, (N, K))
+    b32 = r.integers(-2 ** 31, 2 ** 31, N, dtype=np.int64).astype(np.int32)
+    assert_same(linear_out_32(x, w, b32), oracle.linear_out_32(x, w, b32), "linear_out_32")
+    assert_same(linear_out_32(x, w, None, 64), oracle.linear_out_32(x, w, None), "linear_out_32 no bias")
+
+
+def test_matmul_two_columns():
+    import torch
+    from gpu_helpers import bn_dev, dev
+    r = rng_for(8)
+    K, Co = 27, 7
+    w, cols, b = rand_s8(r, (Co, K)), rand_u8(r, (2, K)), rand_s8(r, (Co,))
+    k, lam = r.integers(256, 1025, Co), r.integers(-2 ** 16, 2 ** 16, Co)
+    w0, w1 = oracle.matmul(w, cols, b, k, lam, 0, 12, 1, 1)
+    L = nn(32)
+    out = torch.zeros(2 * Co + 5, dtype=torch.uint8, device="cuda")
+    ret = L.pulp_nn_matmul(dev(w), dev(cols), Co, K, 12, 0, bn_dev(k, 32), bn_dev(lam, 32), dev(b), out,
+                           out.data_ptr() + Co, 1, 1)
+    L.sync()
+    assert ret == out.data_ptr() + 2 * Co
+    o = out.cpu().numpy()
+    assert_same(o[:Co], w0, "matmul col 0")
+    assert_same(o[Co:2 * Co], w1, "matmul col 1")
+    # separate destinations
+    o2 = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    L.pulp_nn_matmul(dev(w), dev(cols), Co, K, 12, 0, bn_dev(k, 32), bn_dev(lam, 32), dev(b), o2,
+                     o2.data_ptr() + 32, 1, 1)
+    L.sync()
+    o2 = o2.cpu().numpy()
+    assert_same(o2[:Co], w0, "matmul col 0 (split)")
+    assert_same(o2[32:32 + Co], w1, "matmul col 1 (split)")
+
+
+@pytest.mark.parametrize("case", [
+    (2, 63, 63, 256, (2, 2), (2, 2), (32, 32)),    # config 4: ceil mode
+    (2, 63, 63, 16, (2, 2), (2, 2), (31, 31)),
+    (1, 8, 8, 5, (2, 2), (2, 2), (4, 4)),
+    (2, 9, 7, 3, (3, 2), (2, 1), (8, 3)),
+    (1, 6, 6, 4, (3, 3), (3, 3), (2, 2)),
+])
+def test_maxpool(case):
+    B, H, W, Cc, kernel, strides, out_hw = case
+    r = rng_for(7000 + H)
+    x = rand_u8(r, (B, H, W, Cc))
+    got, xin_after = maxpool(x, kernel, strides, out_hw)
+    assert_same(got, oracle.maxpool(x, kernel, strides, out_hw=out_hw), "maxpool")
+    assert_same(xin_after, x, "maxpool input must stay intact")
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+def test_avgpool(bn_bits):
+    r = rng_for(8000)
+    x = rand_u8(r, (3, 4, 4, 512))
+    assert_same(avgpool(x, (4, 4), (4, 4), (1, 1), bn_bits=bn_bits),
+                oracle.avgpool(x, (4, 4), (4, 4), bn_bits=bn_bits), "global avgpool")
+    x2 = rand_u8(r, (2, 9, 7, 6))
+    for pads, kernel, strides, out_hw in [((0, 0, 0, 0), (2, 2), (2, 2), (4, 3)), ((1, 1, 1, 1), (3, 3), (1, 1), (9, 7)),
+                                          ((1, 0, 0, 1), (3, 2), (2, 1), (8, 3))]:
+        for rq, lam, sh, ad in [(0, 0, 0, 0), (1, 3, 2, 20), (1, -1, 22 if bn_bits == 32 else 2, 500)]:
+            want = oracle.avgpool(x2, kernel, strides, pads, out_hw, lam, sh, ad, rq, bn_bits)
+            got = avgpool(x2, kernel, strides, out_hw, pads, lam, sh, ad, rq, bn_bits)
+            assert_same(got, want, "avgpool %s %s" % (pads, (rq, lam)))
+
+
+def test_add():
+    r = rng_for(9000)
+    for shape in [(3, 5, 7, 4), (2, 16, 16, 64), (1, 3, 3, 5)]:
+        a, b = rand_u8(r, shape), rand_u8(r, shape)
+        for m1, m2, d in [(3, 5, 2), (120, 130, 8), (65535, 2, 0), (32767, 32767, 9)]:
+            assert_same(add(a, b, m1, m2, d), oracle.add(a, b, m1, m2, d), "add %s" % ((m1, m2, d),))
+
+
+def test_hwc_to_chw():
+    import torch
+    from gpu_helpers import dev
+    r = rng_for(9100)
+    for B, H, W, Cc, pt, pb in [(2, 7, 9, 5, 1, 1), (1, 16, 16, 64, 0, 0), (3, 5, 4, 130, 1, 0)]:
+        x = rand_u8(r, (B, H, W, Cc))
+        L = nn(32)
+        out = torch.full((B, Cc, H + pt + pb, W), 0xA5, dtype=torch.uint8, device="cuda")
+        L.set_batch(B)
+        L.hwc_to_chw(dev(x), out, W, H, Cc, pt, pb)
+        L.sync()
+        L.set_batch(1)
+        want = np.pad(x.transpose(0, 3, 1, 2), ((0, 0), (0, 0), (pt, pb), (0, 0)))
+        assert_same(out.cpu().numpy(), want, "hwc_to_chw")
+
+
+def test_rejected_calls_report_an_error_and_write_nothing():
+    import torch
+    from pulp_nn_amd import PulpNNError
+    L = nn(32)
+    x = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    out = torch.full((64,), 0xA5, dtype=torch.uint8, device="cuda")
+    w = torch.zeros(64, dtype=torch.int8, device="cuda")
+    with pytest.raises(PulpNNError):   # shift 40 is undefined behaviour for a 32-bit accumulator
+        L.pulp_nn_pointwise_HoWo_parallel(x, None, None, out, w, None, None, 1, 40, 2, 2, 4, 2, 2, 4, 1, 1,
+                                          0, 0, 0, 0, 1, 1, 0, 0)
+    with pytest.raises(PulpNNError):   # batch-norm branch without k / lambda
+        L.pulp_nn_linear(x, None, out, w, None, None, 1, 3, 8, 4, 1, 1)
+    with pytest.raises(PulpNNError):   # p_l = 0: the reference's row pointers drift
+        L.pulp_nn_depthwise_3x3_s1(x, out, 4, 4, 1, 0, 1, w, 3, 1, None, None, 0, 0, None)
+    L.sync()
+    assert int(out.min()) == 0xA5
+    assert L.last_error() == 0
