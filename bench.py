@@ -236,7 +236,7 @@ def main():
                              nthreads=threads)
             reps += 1
             el = time.perf_counter() - t0
-            if el > 10.0 or reps >= 50:
+            if el > 12.0:
                 break
         cpu_gops = (c1["ops"] / 256 * n_img * reps) / el / 1e9
         rec["cpu_baseline"] = {

@@ -82,6 +82,6 @@ def config4(batch=64, relu=1):
         x=_u8(r, (batch, 64, 64, 256)), out_hw=(63, 63),
         lin_w=_s8(r, (4096, 1024)), lin_bias=_s8(r, (4096,)),
         lin_k=r.integers(2 ** 20, 2 ** 24 + 1, 4096).astype(np.int64),
-        lin_lam=r.integers(-2 ** 36, 2 ** 36 + 1, 4096).astype(np.int64), lin_shift=36,
+        lin_lam=r.integers(-2 ** 36, 2 ** 36 + 1, 4096).astype(np.int64), lin_shift=30,
         ops=2 * batch * 63 * 63 * 256 * 2304,
         bytes=batch * (64 * 64 * 256 + 63 * 63 * 256) + 256 * 2304 + 256 * 17)
