@@ -129,16 +129,22 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
   }
 
   v4i areg[RA], wreg[RW];
+  unsigned amask = 0, wmask = 0;  // bit i: chunk i holds real data (else it is staged as zero)
 
+  // Issue the global loads of the next K slice.  Nothing here consumes a loaded value
+  // (that would make the wave wait for it): out-of-image taps and out-of-range rows
+  // load from a clamped, always valid address and are zeroed when staged into LDS.
   auto gload = [&]() {
-    // activations
+    amask = 0;
+    wmask = 0;
 #pragma unroll
     for (int i = 0; i < RA; i++) {
-      v4i v = {0, 0, 0, 0};
       if (GATHER == GATHER_CHUNK16) {
         const int iy = iy0[i] + fy, ix = ix0[i] + fx;
-        if (kpos < g.K && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
-          v = *(const v4i *)(g.in + abase[i] + ((long long)iy * g.W + ix) * g.Ci + ci);
+        const bool ok = kpos < g.K && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+        const long long off = ok ? abase[i] + ((long long)iy * g.W + ix) * g.Ci + ci : 0;
+        areg[i] = *(const v4i *)(g.in + off);
+        amask |= (unsigned)ok << i;
       } else {
         int bfy = fy, bfx = fx, bci = ci;
         unsigned bytes[4] = {0, 0, 0, 0};
@@ -154,32 +160,29 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
             if (++bfx == g.kx) { bfx = 0; ++bfy; }
           }
         }
-        v = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
+        areg[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
+        amask |= 1u << i;
       }
-      areg[i] = v ^ (int)0x80808080;
     }
-    // weights
 #pragma unroll
     for (int i = 0; i < RW; i++) {
-      v4i v = {0, 0, 0, 0};
       const int n = n0 + wchan[i];
-      if (wact[i] && n < g.N) {
-        const int8_t *src = g.w + (long long)n * g.K + kpos;
-        if (GATHER == GATHER_CHUNK16) {
-          if (kpos < g.K) v = *(const v4i *)src;
-        } else {
-          unsigned bytes[4] = {0, 0, 0, 0};
+      if (GATHER == GATHER_CHUNK16) {
+        const bool ok = wact[i] && n < g.N && kpos < g.K;
+        const long long off = ok ? (long long)n * g.K + kpos : 0;
+        wreg[i] = *(const v4i *)(g.w + off);
+        wmask |= (unsigned)ok << i;
+      } else {
+        unsigned bytes[4] = {0, 0, 0, 0};
+        if (wact[i] && n < g.N) {
+          const int8_t *src = g.w + (long long)n * g.K + kpos;
 #pragma unroll
           for (int j = 0; j < 16; j++)
             if (kpos + j < g.K) bytes[j >> 2] |= (unsigned)(uint8_t)src[j] << (8 * (j & 3));
-          v = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
         }
+        wreg[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
+        wmask |= 1u << i;
       }
-      wreg[i] = v;
-      wpart[i] = __builtin_amdgcn_sdot4(v.x, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.y, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.z, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.w, 0x01010101, wpart[i], false);
     }
     // advance to the next K slice
     kpos += IGEMM_BK;
@@ -190,13 +193,25 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
     }
   };
 
+  // Stage the loaded slice into LDS: activations as a ^ 0x80, invalid chunks as zero
+  // (0x80 after the xor); weight bytes also feed the per-row sums.
   auto sts = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < RA; i++)
-      *(v4i *)&As[buf][lds_off((tid >> 2) + 64 * i, ck)] = areg[i];
+    for (int i = 0; i < RA; i++) {
+      v4i v = areg[i];
+      if (!((amask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      *(v4i *)&As[buf][lds_off((tid >> 2) + 64 * i, ck)] = v ^ (int)0x80808080;
+    }
 #pragma unroll
-    for (int i = 0; i < RW; i++)
-      if (wact[i]) *(v4i *)&Ws[buf][lds_off(wrow[i], ck)] = wreg[i];
+    for (int i = 0; i < RW; i++) {
+      v4i v = wreg[i];
+      if (!((wmask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      if (wact[i]) *(v4i *)&Ws[buf][lds_off(wrow[i], ck)] = v;
+      wpart[i] = __builtin_amdgcn_sdot4(v.x, 0x01010101, wpart[i], false);
+      wpart[i] = __builtin_amdgcn_sdot4(v.y, 0x01010101, wpart[i], false);
+      wpart[i] = __builtin_amdgcn_sdot4(v.z, 0x01010101, wpart[i], false);
+      wpart[i] = __builtin_amdgcn_sdot4(v.w, 0x01010101, wpart[i], false);
+    }
   };
 
   v4i acc[TN][TM];

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #if PULPNN_BN_BITS == 64
 #include "../../include/64bit/pulp_nn_kernels.h"
@@ -18,6 +19,7 @@
 #include "depthwise.h"
 #include "igemm.h"
 #include "pool.h"
+#include "pw_stream.h"
 #include "requant.h"
 
 namespace {
@@ -101,6 +103,96 @@ void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
 }
 
+int num_cus()
+{
+  static int n = 0;
+  if (!n) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
+template <int TN, int KS>
+void launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
+{
+  constexpr int TM = 2;
+  dim3 block(256);
+  switch (mode) {
+    case EPI_BN:
+      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_BN, false, TM>), grid, block, lds, s, g, e);
+      break;
+    case EPI_MULT:
+      if (e.shift >= 16)
+        hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_MULT, true, TM>), grid, block, lds, s, g, e);
+      else
+        hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_MULT, false, TM>), grid, block, lds, s, g, e);
+      break;
+    case EPI_RAW:
+      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_RAW, false, TM>), grid, block, lds, s, g, e);
+      break;
+    default:
+      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_OUT32, false, TM>), grid, block, lds, s, g, e);
+      break;
+  }
+}
+
+template <int TN>
+void launch_pw_stream_ks(int mode, int ks, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
+{
+  if (ks == 1) launch_pw_stream_mode<TN, 1>(mode, g, e, grid, lds, s);
+  else if (ks == 2) launch_pw_stream_mode<TN, 2>(mode, g, e, grid, lds, s);
+  else launch_pw_stream_mode<TN, 4>(mode, g, e, grid, lds, s);
+}
+
+// Weights-stationary streaming path: a GEMM whose rows are contiguous K-byte pixels,
+// whose weight matrix (at most 256 x 256) fits in LDS and whose channel count is one
+// of 16, 32, 64, 128, 192, 256 (every lane then owns real channels and stores whole
+// vectors).  Returns false if the shape does not qualify (the caller then uses the
+// tiled kernel).
+bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *bias, void *out, long long M, int N,
+                   int K, const EpiArgs &e, hipStream_t s)
+{
+  if (K > 256 || (K % 16) || !aligned(in, 16) || !aligned(w, 16) || !aligned(out, 16) || M < 2048) return false;
+  if (!(N == 16 || N == 32 || N == 64 || N == 128 || N == 192 || N == 256)) return false;
+  if (mode == EPI_OUT32) return false;
+  const int tn = N == 16 ? 1 : (N == 32 ? 2 : 4);
+  const int np = N / (16 * tn);
+  const int ks = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
+  constexpr int tm = 2;
+  PwGeom g;
+  g.in = in;
+  g.w = w;
+  g.bias = bias;
+  g.out = out;
+  g.M = (int)M;
+  g.N = N;
+  g.K = K;
+  const int lds = pw_lds_bytes(tn, ks, np, mode == EPI_BN);
+  if (lds > 65536) return false;
+  g.pgroups = (int)((M + 16 * tm - 1) / (16 * tm));
+  // Persistent grid: as many workgroups as stay resident, then trimmed so that every
+  // wave runs the same number of steps.
+  static const char *capenv = getenv("PULPNN_CAP");
+  int per_cu = 163840 / lds;
+  const int per_cu_max = capenv ? atoi(capenv) : 4;
+  if (per_cu > per_cu_max) per_cu = per_cu_max;
+  const int cap = per_cu * num_cus();
+  int blocks = (g.pgroups + 3) / 4;
+  if (blocks > cap) {
+    const int steps = (blocks + cap - 1) / cap;
+    blocks = (blocks + steps - 1) / steps;
+  }
+  dim3 grid(blocks);
+  g.npass = np;
+  if (tn == 1) launch_pw_stream_ks<1>(mode, ks, g, e, grid, lds, s);
+  else if (tn == 2) launch_pw_stream_ks<2>(mode, ks, g, e, grid, lds, s);
+  else launch_pw_stream_ks<4>(mode, ks, g, e, grid, lds, s);
+  return true;
+}
+
 // Shared body of the six convolution entry points.
 void conv_common(const char *fn, bool pointwise, const uint8_t *in, const int8_t *bias, uint8_t *out,
                  const int8_t *w, bn_t *k, bn_t *lambda, uint16_t out_mult, uint16_t out_shift,
@@ -127,6 +219,11 @@ void conv_common(const char *fn, bool pointwise, const uint8_t *in, const int8_t
     return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "out_shift out of range or null k/lambda");
   const long long M = (long long)g_batch * dim_out_x * dim_out_y;
   if (M > 0x7fffffffLL) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+  if (kx == 1 && ky == 1 && sx == 1 && sy == 1 && pt == 0 && pl == 0 && dim_out_x == dim_in_x &&
+      dim_out_y == dim_in_y && try_pw_stream(mode, in, w, bias, out, M, ch_out, ch_in, e, g_stream)) {
+    check_launch(fn);
+    return;
+  }
   ConvGeom g;
   g.in = in;
   g.w = w;

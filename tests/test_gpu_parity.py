@@ -74,6 +74,15 @@ PW_GEOMS = [
     (2, 4, 4, 512, 512),
     (1, 9, 11, 3, 100),
     (5, 3, 3, 70, 64),
+    # shapes that take the weights-stationary streaming kernel (>= 2048 pixels, K, N <= 256)
+    (4, 32, 32, 16, 32),     # 16 -> 32 channels (MobileNet block 1), K < 64
+    (3, 30, 30, 32, 16),     # N = 16
+    (2, 40, 40, 64, 64),     # one channel group
+    (2, 33, 35, 64, 128),    # two channel groups, pixel count not a multiple of 64
+    (2, 33, 33, 256, 200),   # K = 256, channel tail inside the last group
+    (2, 40, 30, 48, 100),    # K and N not multiples of 64
+    (3, 33, 33, 192, 256),   # K = 192
+    (1, 50, 50, 128, 20),    # N not a multiple of 16
 ]
 
 
