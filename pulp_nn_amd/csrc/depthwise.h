@@ -24,6 +24,8 @@
 #pragma once
 #include "requant.h"
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+
 struct DwGeom {
   const uint8_t *in;
   const int8_t *wt;
@@ -98,6 +100,19 @@ __device__ __forceinline__ unsigned quad_transpose4x4(unsigned v, int lane)
   t = (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true);
   v = (lane & 1) ? (((t >> 8) & 0x00FF00FFu) | (v & 0xFF00FF00u)) : ((v & 0x00FF00FFu) | ((t << 8) & 0xFF00FF00u));
   return v;
+}
+
+// The same transpose with v_perm_b32: sel1 / sel2 are per-lane byte selectors
+// (quad_sel1 / quad_sel2 of the lane), so there is no per-lane branch or select.
+// v_perm_b32 D, S0, S1, sel: selector values 0-3 pick bytes of S1, 4-7 bytes of S0.
+__device__ __forceinline__ unsigned quad_sel1(int lane) { return (lane & 2) ? 0x03020706u : 0x05040100u; }
+__device__ __forceinline__ unsigned quad_sel2(int lane) { return (lane & 1) ? 0x03070105u : 0x06020400u; }
+__device__ __forceinline__ unsigned quad_transpose4x4_perm(unsigned v, unsigned sel1, unsigned sel2)
+{
+  unsigned t = (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true);
+  v = __builtin_amdgcn_perm(t, v, sel1);
+  t = (unsigned)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true);
+  return __builtin_amdgcn_perm(t, v, sel2);
 }
 
 // bytes [o, o+4) of the little-endian byte string formed by the dwords of `span`
@@ -206,6 +221,242 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(DwGeom g, EpiArgs e)
         for (int c = 0; c < 4; c++)
           if (c0 + cq + c < g.CH) o[c] = (uint8_t)(packed >> (8 * c));
       }
+    }
+  }
+}
+
+// One group of 4 output columns of one channel per lane, walked down the rows of a band.
+struct DwColumn {
+  const unsigned *p;  // LDS: first dword of the window in the first staged row
+  uint8_t *o;         // output byte of the first row for this lane (after the quad transpose)
+  long long row_bytes;
+  int LWD, dc0, rows;
+  int corr, mult, shift;
+  bn_t k, lambda;
+  unsigned wA[3], wB[3], sel1, sel2;
+  int store, nbytes;
+};
+
+template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ>
+__device__ __forceinline__ void dw3x3_column(DwColumn c)
+{
+  constexpr int O0 = 4 - PL;
+  constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
+  bool in_row[NS];
+#pragma unroll
+  for (int d = 0; d < NS; d++) in_row[d] = !EDGE || (c.dc0 + d >= 0 && c.dc0 + d < c.LWD);
+  auto read_row = [&](unsigned (&span)[NS]) {
+#pragma unroll
+    for (int d = 0; d < NS; d++) span[d] = in_row[d] ? c.p[d] : 0x80808080u;
+    c.p += c.LWD;
+  };
+  // K_i . window_j of one input row, for the four output columns j
+  auto taps = [&](const unsigned (&span)[NS], int i, int (&acc)[4]) {
+    dw_tap<O0, NS>(span, c.wA[i], c.wB[i], acc[0]);
+    dw_tap<O0 + S, NS>(span, c.wA[i], c.wB[i], acc[1]);
+    dw_tap<O0 + 2 * S, NS>(span, c.wA[i], c.wB[i], acc[2]);
+    dw_tap<O0 + 3 * S, NS>(span, c.wA[i], c.wB[i], acc[3]);
+  };
+  auto emit = [&](int (&acc)[4]) {
+    unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], c.k, c.lambda, c.mult, c.shift);
+    packed = quad_transpose4x4_perm(packed, c.sel1, c.sel2);
+    if constexpr (FULL) {
+      *(unsigned *)c.o = packed;
+    } else {
+      if (c.store == 0) {
+        *(unsigned *)c.o = packed;
+      } else if (c.store == 1) {
+        for (int j = 0; j < c.nbytes; j++) c.o[j] = (uint8_t)(packed >> (8 * j));
+      }
+    }
+    c.o += c.row_bytes;
+  };
+
+  unsigned span[NS];
+  if constexpr (S == 1) {
+    // P: output row y-2 so far (K0, K1 rows done); Q: output row y-1 so far (K0 done)
+    int P[4], Q[4];
+    read_row(span);
+#pragma unroll
+    for (int j = 0; j < 4; j++) P[j] = c.corr;
+    taps(span, 0, P);
+    read_row(span);
+#pragma unroll
+    for (int j = 0; j < 4; j++) Q[j] = c.corr;
+    taps(span, 1, P);
+    taps(span, 0, Q);
+    for (int r = 0; r < c.rows; r++) {
+      read_row(span);
+      taps(span, 2, P);
+      emit(P);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        P[j] = Q[j];
+        Q[j] = c.corr;
+      }
+      taps(span, 1, P);
+      taps(span, 0, Q);
+    }
+  } else {
+    // Q: next output row so far (K0 row done)
+    int Q[4];
+    read_row(span);
+#pragma unroll
+    for (int j = 0; j < 4; j++) Q[j] = c.corr;
+    taps(span, 0, Q);
+    for (int r = 0; r < c.rows; r++) {
+      read_row(span);
+      taps(span, 1, Q);
+      read_row(span);
+      taps(span, 2, Q);
+      emit(Q);
+#pragma unroll
+      for (int j = 0; j < 4; j++) Q[j] = c.corr;
+      taps(span, 0, Q);
+    }
+  }
+}
+
+// 3x3 depthwise, fast variant for W % 4 == 0 and a 16-byte aligned input.
+//
+// LDS holds the band exactly as it lies in memory (rows of W bytes back to back,
+// no column padding), so staging is a linear copy: each wave copies the
+// contiguous run of each of its 16 channels with one 16-byte load per lane, all
+// loads in flight before the first LDS write.  The columns left of 0 and right
+// of W-1 are supplied in the compute phase instead: a wave works on one group of
+// 4 output columns at a time and walks down the rows of the band, so whether a
+// dword of the 3-dword window lies outside the row is decided once per column
+// group; outside dwords are replaced by 0x80808080 (a = 0).  Walking down the rows
+// also means every input dword is read from LDS once, not three times: the three
+// partial sums an input row contributes to are kept in registers.
+//
+// FULL: Wo % 4 == 0, CH % 64 == 0 and the output is 4-byte aligned, so every lane
+// stores one dword per output row without any bounds check.
+template <int S, int PL, int MODE, bool FULL>
+__global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
+{
+  extern __shared__ unsigned dw_lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  int id = dw_xcd_remap(blockIdx.x, g.total);
+  const int cg = id % g.cgroups;
+  id /= g.cgroups;
+  const int band = id % g.bands;
+  const int b = id / g.bands;
+  const int c0 = cg * DW_CG;
+  const int oy0 = band * g.RB;
+  const int rows = min(g.RB, g.Ho - oy0);
+  const int iy_start = oy0 * S - g.pt;
+  const int LWD = g.LWD;  // = W / 4
+  const int dummy = DW_CG * g.CSD;  // one spare dword behind the tile: target of masked-off writes
+
+  // ---- stage -----------------------------------------------------------------
+  const int r_lo = max(0, -iy_start), r_hi = min(g.NR, g.H - iy_start);  // rows of the band inside the image
+  const int run_len = max(r_hi - r_lo, 0) * g.W;                        // bytes per channel
+  const uint8_t *img = g.in + (long long)b * g.CH * g.H * g.W;
+  const bool two = run_len + 12 > 64 * 16;  // a run may need more than 64 chunks
+  {
+    v4i ld[16][2];
+    int mis[16];
+#pragma unroll
+    for (int cc = 0; cc < 16; cc++) {
+      const int ch = min(c0 + wave + 4 * cc, g.CH - 1);
+      const uint8_t *g0 = img + ((long long)ch * g.H + min(max(iy_start + r_lo, 0), g.H - 1)) * g.W;
+      mis[cc] = (int)((uintptr_t)g0 & 15);
+      const int last = max(((run_len + mis[cc] + 15) >> 4) - 1, 0);
+      // lanes past the end of the run re-read its last chunk (masked off below)
+      ld[cc][0] = *(const v4i *)(g0 - mis[cc] + 16 * min(lane, last));
+      if (two) ld[cc][1] = *(const v4i *)(g0 - mis[cc] + 16 * min(lane + 64, last));
+    }
+#pragma unroll
+    for (int cc = 0; cc < 16; cc++) {
+      const int c = wave + 4 * cc;
+      const int dst = c * g.CSD + r_lo * LWD;
+      const unsigned keep = (c0 + c < g.CH) ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        if (t == 1 && !two) break;
+        const int o = 16 * (lane + 64 * t) - mis[cc];  // byte offset of this chunk in the run
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int ob = o + 4 * u;
+          const bool ok = ob >= 0 && ob < run_len;
+          dw_lds[ok ? dst + (ob >> 2) : dummy] = ((unsigned)ld[cc][t][u] & keep) ^ 0x80808080u;
+        }
+      }
+      // rows of the band above / below the image
+      unsigned *base = dw_lds + c * g.CSD;
+      for (int q = lane; q < r_lo * LWD; q += 64) base[q] = 0x80808080u;
+      for (int q = r_hi * LWD + lane; q < g.NR * LWD; q += 64) base[q] = 0x80808080u;
+    }
+  }
+
+  // ---- per-lane channel constants ------------------------------------------------
+  const int ch = c0 + lane;
+  const bool ch_ok = ch < g.CH;
+  unsigned wA[3], wB[3];
+  int corr = 0;
+  bn_t kk = 0, ll = 0;
+  if (ch_ok) {
+    int wsum = 0;
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      const int8_t *p = g.wt + (long long)ch * 9 + 3 * i;
+      const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
+      wA[i] = k0 | (k1 << 8) | (k2 << 16);
+      wB[i] = wA[i] << 8;
+      wsum += (int)p[0] + (int)p[1] + (int)p[2];
+    }
+    corr = 128 * wsum + (g.bias ? (int)g.bias[ch] : 0);
+    if (MODE == EPI_BN) {
+      kk = e.k[ch];
+      ll = e.lambda[ch];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; i++) wA[i] = wB[i] = 0;
+  }
+  const bool k_small = __all(bn_k_small(kk));
+  __syncthreads();
+
+  // ---- compute -------------------------------------------------------------------------
+  const int xgroups = (g.Wo + 3) >> 2;
+  const unsigned *lbase = dw_lds + lane * g.CSD - 1;
+  DwColumn col;
+  col.LWD = LWD;
+  col.rows = rows;
+  col.row_bytes = (long long)g.Wo * g.CH;
+  col.corr = corr;
+  col.k = kk;
+  col.lambda = ll;
+  col.mult = e.mult;
+  col.shift = e.shift;
+  col.sel1 = quad_sel1(lane);
+  col.sel2 = quad_sel2(lane);
+#pragma unroll
+  for (int i = 0; i < 3; i++) {
+    col.wA[i] = wA[i];
+    col.wB[i] = wB[i];
+  }
+  const int cq = lane & ~3;
+  const bool fastq = (MODE == EPI_BN) ? k_small : (e.shift >= 16);
+  constexpr int NS = ((4 - PL) + 3 * S + 2) / 4 + 1;
+
+  for (int xg = wave; xg < xgroups; xg += 4) {
+    col.dc0 = xg * S - 1;  // dword column of the first dword of the window
+    col.p = lbase + xg * S;
+    col.o = g.out + (((long long)b * g.Ho + oy0) * g.Wo + 4 * xg + (lane & 3)) * g.CH + c0 + cq;
+    // 0: store a dword, 1: store the valid bytes one by one, 2: nothing to store
+    col.store = (4 * xg + (lane & 3) >= g.Wo) ? 2 : ((g.out_vec4 && c0 + cq + 3 < g.CH) ? 0 : 1);
+    col.nbytes = min(4, g.CH - c0 - cq);
+    const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
+    if (fastq) {
+      if (edge) dw3x3_column<S, PL, MODE, FULL, true, true>(col);
+      else dw3x3_column<S, PL, MODE, FULL, false, true>(col);
+    } else {
+      if (edge) dw3x3_column<S, PL, MODE, FULL, true, false>(col);
+      else dw3x3_column<S, PL, MODE, FULL, false, false>(col);
     }
   }
 }

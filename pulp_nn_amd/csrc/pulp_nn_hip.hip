@@ -306,6 +306,9 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.sx = sx;
   g.sy = sy;
   const bool fast = kx == 3 && ky == 3 && sx == sy && (sx == 1 || sx == 2) && (pl == 0 || pl == 1);
+  // linear variant: LDS rows are the image rows themselves (W / 4 dwords, no padding)
+  static const char *nolin = getenv("PULPNN_DW_NOLIN");
+  const bool lin = fast && (W % 4 == 0) && aligned(in, 16) && W / 4 * 3 <= 255 && !nolin;
   g.LP = pl > 4 ? ((pl + 3) & ~3) : 4;
   int need_bytes;  // bytes of an LDS row the compute phase may touch
   if (fast) {
@@ -317,6 +320,10 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   }
   const int img_bytes = g.LP + W + 1;
   g.LWD = ((need_bytes > img_bytes ? need_bytes : img_bytes) + 3) / 4;
+  if (lin) {
+    g.LP = 0;
+    g.LWD = W / 4;
+  }
   const int max_csd = 255;  // 64 channels x 255 dwords = 63.75 KiB of LDS
   int nr_max = max_csd / g.LWD;
   if (nr_max < ky) return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "image too wide for the LDS tile");
@@ -346,7 +353,28 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     default: hipLaunchKernelGGL((KERNEL<EPI_RAW>), grid, block, lds, g_stream, g, e); break;        \
   }
 #define DW3(S, PL, M) dw3x3_kernel<S, PL, M>
-  if (fast) {
+  if (lin) {
+    const bool full = (Wo % 4 == 0) && (CH % DW_CG == 0) && g.out_vec4;
+    const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
+#define DW3L_MODE(S, PL, FULL)                                                                                        \
+  switch (mode) {                                                                                                     \
+    case EPI_BN: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_BN, FULL>), grid, block, ldsl, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_MULT, FULL>), grid, block, ldsl, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_RAW, FULL>), grid, block, ldsl, g_stream, g, e); break;        \
+  }
+#define DW3L(S, PL)          \
+  if (full) {                \
+    DW3L_MODE(S, PL, true)   \
+  } else {                   \
+    DW3L_MODE(S, PL, false)  \
+  }
+    if (sx == 1 && pl == 1) { DW3L(1, 1) }
+    else if (sx == 1) { DW3L(1, 0) }
+    else if (pl == 1) { DW3L(2, 1) }
+    else { DW3L(2, 0) }
+#undef DW3L
+#undef DW3L_MODE
+  } else if (fast) {
     if (sx == 1 && pl == 1) { switch (mode) {
       case EPI_BN: hipLaunchKernelGGL((DW3(1, 1, EPI_BN)), grid, block, lds, g_stream, g, e); break;
       case EPI_MULT: hipLaunchKernelGGL((DW3(1, 1, EPI_MULT)), grid, block, lds, g_stream, g, e); break;

@@ -185,3 +185,47 @@ __device__ __forceinline__ bool bn_k_small(bn_t k)
   return k >= -(1 << 23) && k < (1 << 23);
 #endif
 }
+
+// Four outputs of ONE channel (depthwise); |acc| < 2^23.  The accumulators come from
+// v_dot4 instructions, so everything that reads them directly is compiler-visible code
+// (the inline-asm pack only ever sees results of ordinary VALU instructions).
+// FASTQ: batch-norm branch: k fits 24 bits (32-bit build) / 32 bits (64-bit build);
+//        multiplier branch: shift >= 16 (the int16 narrowing is then the identity).
+template <int MODE, bool FASTQ>
+__device__ __forceinline__ unsigned requant4_same(int a0, int a1, int a2, int a3, bn_t k, bn_t lambda, int mult,
+                                                  int shift)
+{
+  if constexpr (MODE == EPI_RAW) {
+    return ashr_sat_pack4_safe(a0, a1, a2, a3, shift);
+  } else if constexpr (MODE == EPI_MULT) {
+    int p0 = __mul24(a0, mult), p1 = __mul24(a1, mult), p2 = __mul24(a2, mult), p3 = __mul24(a3, mult);
+    if constexpr (FASTQ) return ashr_sat_pack4(p0, p1, p2, p3, shift);
+    p0 = (int)(short)(p0 >> shift);
+    p1 = (int)(short)(p1 >> shift);
+    p2 = (int)(short)(p2 >> shift);
+    p3 = (int)(short)(p3 >> shift);
+    return ashr_sat_pack4(p0, p1, p2, p3, 0);
+  } else {
+#if PULPNN_BN_BITS == 64
+    const bn_t kk[4] = {k, k, k, k}, ll[4] = {lambda, lambda, lambda, lambda};
+    return requant4<EPI_BN, true>(a0, a1, a2, a3, kk, ll, FASTQ, mult, shift);
+#else
+    int v0, v1, v2, v3;
+    if constexpr (FASTQ) {
+      // compiler-visible multiplies: the accumulators come from v_dot4, whose results
+      // other VALU instructions may only read after wait states the compiler inserts
+      const int k32 = (int)k, l32 = (int)lambda;
+      v0 = __mul24(a0, k32) + l32;
+      v1 = __mul24(a1, k32) + l32;
+      v2 = __mul24(a2, k32) + l32;
+      v3 = __mul24(a3, k32) + l32;
+    } else {
+      v0 = (int)((unsigned)k * (unsigned)a0 + (unsigned)lambda);
+      v1 = (int)((unsigned)k * (unsigned)a1 + (unsigned)lambda);
+      v2 = (int)((unsigned)k * (unsigned)a2 + (unsigned)lambda);
+      v3 = (int)((unsigned)k * (unsigned)a3 + (unsigned)lambda);
+    }
+    return ashr_sat_pack4(v0, v1, v2, v3, shift);
+#endif
+  }
+}
