@@ -175,10 +175,8 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   g.pgroups = (int)((M + 16 * tm - 1) / (16 * tm));
   // Persistent grid: as many workgroups as stay resident, then trimmed so that every
   // wave runs the same number of steps.
-  static const char *capenv = getenv("PULPNN_CAP");
   int per_cu = 163840 / lds;
-  const int per_cu_max = capenv ? atoi(capenv) : 4;
-  if (per_cu > per_cu_max) per_cu = per_cu_max;
+  if (per_cu > 2) per_cu = 2;  // measured: more resident workgroups do not stream faster
   const int cap = per_cu * num_cus();
   int blocks = (g.pgroups + 3) / 4;
   if (blocks > cap) {
@@ -307,8 +305,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.sy = sy;
   const bool fast = kx == 3 && ky == 3 && sx == sy && (sx == 1 || sx == 2) && (pl == 0 || pl == 1);
   // linear variant: LDS rows are the image rows themselves (W / 4 dwords, no padding)
-  static const char *nolin = getenv("PULPNN_DW_NOLIN");
-  const bool lin = fast && (W % 4 == 0) && aligned(in, 16) && W / 4 * 3 <= 255 && !nolin;
+  const bool lin = fast && (W % 4 == 0) && aligned(in, 16) && W / 4 * 3 <= 255;
   g.LP = pl > 4 ? ((pl + 3) & ~3) : 4;
   int need_bytes;  // bytes of an LDS row the compute phase may touch
   if (fast) {
