@@ -124,7 +124,7 @@ def main():
         "mfma_frac": round(c1["ops"] / (dev_ms * 1e-3) / PEAK_INT8_OPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "igemm_kernel (pointwise, 128x128 tile, scalar-multiplier epilogue)",
+            "kernel": "pw_stream_kernel<4, 2, 1, true, 2> (weights-stationary pointwise, scalar-multiplier epilogue)",
             "achieved": round(c1["bytes"] / (dev_ms * 1e-3) / 1e9, 1),
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
@@ -220,7 +220,51 @@ def main():
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
         layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev,
                      np.array_equal(outs4[0][:1].cpu().numpy(), want))
-        del xs4, outs4
+        # the rest of configuration 4: maxpool 2x2 s2 (63 -> 32) and the 1024 -> 4096 linear layer
+        pooled = [torch.zeros((64, 32, 32, 256), dtype=torch.uint8, device="cuda") for _ in range(nset)]
+
+        def step_mp(i):
+            j = i % nset
+            L4.pulp_nn_maxpool(outs4[j], pooled[j], 63, 63, 256, 32, 32, 2, 2, 0, 0, 0, 0, 2, 2)
+
+        wall, dev = time_launches(step_mp, steps, warm)
+        want = oracle.maxpool(outs4[0][:2].cpu().numpy(), (2, 2), (2, 2), out_hw=(32, 32))
+        mp_bytes = 64 * (63 * 63 * 256 + 32 * 32 * 256)
+        layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev,
+                     np.array_equal(pooled[0][:2].cpu().numpy(), want))
+        vec = torch.randint(0, 255, (64, 1024), dtype=torch.uint8, device="cuda")
+        lw, lb, lk, ll = t(c4["lin_w"]), t(c4["lin_bias"]), t(c4["lin_k"]), t(c4["lin_lam"])
+        lout = torch.zeros((64, 4096), dtype=torch.uint8, device="cuda")
+
+        def step_lin(i):
+            L4.pulp_nn_linear(vec, lb, lout, lw, lk, ll, 0, c4["lin_shift"], 1024, 4096, 1, 1)
+
+        wall, dev = time_launches(step_lin, steps, warm)
+        want = oracle.linear(vec.cpu().numpy(), c4["lin_w"], c4["lin_bias"], c4["lin_k"], c4["lin_lam"], 0,
+                             c4["lin_shift"], 1, 1, 64)
+        layer_record("cfg4_linear_1024_4096_b64", 2 * 64 * 1024 * 4096, 64 * (1024 + 4096) + 4096 * 1024 + 4096 * 17,
+                     wall, dev, np.array_equal(lout.cpu().numpy(), want))
+        del xs4, outs4, pooled
+
+        # configuration 3: the whole MobileNetV1-0.5 chain at batch 256 (29 layer launches + 13 layout changes)
+        from pulp_nn_amd import mobilenet
+        net = mobilenet.build(256)
+        runner = mobilenet.Runner(libs[32], net)
+        x3 = t(net["x"])
+
+        def step_net(i):
+            runner.run(x3)
+
+        wall, dev = time_launches(step_net, max(5, steps // 4), 2)
+        libs[32].sync()
+        import hashlib
+        dig = json.load(open(os.path.join(ROOT, "tests", "golden", "config_digests.json")))["cfg3_b256_logits"]["sha256"]
+        ok = hashlib.sha256(runner.logits.cpu().numpy().tobytes()).hexdigest() == dig
+        layers.append({"layer": "cfg3_mobilenet_v1_0.5_128x128_b256 (whole chain)", "ms": round(dev, 5),
+                       "wall_ms": round(wall, 5), "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
+                       "images_per_s": round(256 / (wall * 1e-3), 1),
+                       "mfma_frac": round(net["ops"] / (dev * 1e-3) / PEAK_INT8_OPS, 4),
+                       "parity": "bit-exact (logits digest)" if ok else "MISMATCH"})
         rec["layers"] = layers
 
     # ---- CPU baseline: the oracle on this machine's host cores --------------------
