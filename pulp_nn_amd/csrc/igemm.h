@@ -48,6 +48,9 @@ struct ConvGeom {
 };
 
 #define IGEMM_BK 64
+#ifndef IGEMM_MINB
+#define IGEMM_MINB 2  // workgroups per CU the register budget is sized for
+#endif
 
 // Tile index of this workgroup.  Workgroups are dealt round-robin to the 8
 // XCDs; the remap gives each XCD a contiguous range of tiles so that tiles
@@ -64,10 +67,9 @@ __device__ __forceinline__ int lds_off(int row, int chunk)
   return row * IGEMM_BK + ((chunk ^ ((row >> 1) & 3)) << 4);
 }
 
-template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE>
-__global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
+template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4>
+__global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiArgs e)
 {
-  constexpr int TM = 4;
   constexpr int WM = 16 * TM, WN = 16 * TN;
   constexpr int BM = WM * WAVES_M, BN = WN * WAVES_N;
   constexpr int RA = BM / 64;                    // activation chunks per thread per K slice
@@ -128,22 +130,26 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
     wpart[i] = 0;
   }
 
-  v4i areg[RA], wreg[RW];
-  unsigned amask = 0, wmask = 0;  // bit i: chunk i holds real data (else it is staged as zero)
+  // Two register sets: the loads of K slice kt+2 are in flight while slice kt is
+  // multiplied and slice kt+1 is staged, so a load has two slices of MFMA work to arrive.
+  struct Staged {
+    v4i a[RA], w[RW];
+    unsigned amask, wmask;  // bit i: chunk i holds real data (else it is staged as zero)
+  };
+  Staged R0, R1;
 
   // Issue the global loads of the next K slice.  Nothing here consumes a loaded value
   // (that would make the wave wait for it): out-of-image taps and out-of-range rows
   // load from a clamped, always valid address and are zeroed when staged into LDS.
-  auto gload = [&]() {
-    amask = 0;
-    wmask = 0;
+  auto gload = [&](Staged &R) {
+    unsigned amask = 0, wmask = 0;
 #pragma unroll
     for (int i = 0; i < RA; i++) {
       if (GATHER == GATHER_CHUNK16) {
         const int iy = iy0[i] + fy, ix = ix0[i] + fx;
         const bool ok = kpos < g.K && (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
         const long long off = ok ? abase[i] + ((long long)iy * g.W + ix) * g.Ci + ci : 0;
-        areg[i] = *(const v4i *)(g.in + off);
+        R.a[i] = *(const v4i *)(g.in + off);
         amask |= (unsigned)ok << i;
       } else {
         int bfy = fy, bfx = fx, bci = ci;
@@ -160,7 +166,7 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
             if (++bfx == g.kx) { bfx = 0; ++bfy; }
           }
         }
-        areg[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
+        R.a[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
         amask |= 1u << i;
       }
     }
@@ -170,7 +176,7 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
       if (GATHER == GATHER_CHUNK16) {
         const bool ok = wact[i] && n < g.N && kpos < g.K;
         const long long off = ok ? (long long)n * g.K + kpos : 0;
-        wreg[i] = *(const v4i *)(g.w + off);
+        R.w[i] = *(const v4i *)(g.w + off);
         wmask |= (unsigned)ok << i;
       } else {
         unsigned bytes[4] = {0, 0, 0, 0};
@@ -180,10 +186,12 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
           for (int j = 0; j < 16; j++)
             if (kpos + j < g.K) bytes[j >> 2] |= (unsigned)(uint8_t)src[j] << (8 * (j & 3));
         }
-        wreg[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
+        R.w[i] = (v4i){(int)bytes[0], (int)bytes[1], (int)bytes[2], (int)bytes[3]};
         wmask |= 1u << i;
       }
     }
+    R.amask = amask;
+    R.wmask = wmask;
     // advance to the next K slice
     kpos += IGEMM_BK;
     ci += IGEMM_BK;
@@ -195,17 +203,17 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
 
   // Stage the loaded slice into LDS: activations as a ^ 0x80, invalid chunks as zero
   // (0x80 after the xor); weight bytes also feed the per-row sums.
-  auto sts = [&](int buf) {
+  auto sts = [&](const Staged &R, int buf) {
 #pragma unroll
     for (int i = 0; i < RA; i++) {
-      v4i v = areg[i];
-      if (!((amask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      v4i v = R.a[i];
+      if (!((R.amask >> i) & 1)) v = (v4i){0, 0, 0, 0};
       *(v4i *)&As[buf][lds_off((tid >> 2) + 64 * i, ck)] = v ^ (int)0x80808080;
     }
 #pragma unroll
     for (int i = 0; i < RW; i++) {
-      v4i v = wreg[i];
-      if (!((wmask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      v4i v = R.w[i];
+      if (!((R.wmask >> i) & 1)) v = (v4i){0, 0, 0, 0};
       if (wact[i]) *(v4i *)&Ws[buf][lds_off(wrow[i], ck)] = v;
       wpart[i] = __builtin_amdgcn_sdot4(v.x, 0x01010101, wpart[i], false);
       wpart[i] = __builtin_amdgcn_sdot4(v.y, 0x01010101, wpart[i], false);
@@ -226,12 +234,7 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
   const int afrag_row0 = wave_m * WM + l16;
 
   const int KT = (g.K + IGEMM_BK - 1) / IGEMM_BK;
-  gload();
-  sts(0);
-  __syncthreads();
-  for (int kt = 0; kt < KT; kt++) {
-    const int cur = kt & 1;
-    if (kt + 1 < KT) gload();
+  auto compute = [&](int cur) {
     v4i wf[TN], af[TM];
 #pragma unroll
     for (int t = 0; t < TN; t++) wf[t] = *(const v4i *)&Ws[cur][lds_off(wfrag_row0 + 16 * t, lgrp)];
@@ -242,7 +245,21 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
 #pragma unroll
       for (int s = 0; s < TM; s++)
         acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[t], af[s], acc[t][s], 0, 0, 0);
-    if (kt + 1 < KT) sts(cur ^ 1);
+  };
+  // Slices past the end load nothing (all-zero masks) and stage zeros: no branches needed.
+  gload(R0);
+  sts(R0, 0);
+  gload(R1);
+  __syncthreads();
+  for (int kt = 0; kt < KT; kt += 2) {
+    gload(R0);        // slice kt + 2
+    compute(0);       // slice kt
+    sts(R1, 1);       // slice kt + 1
+    __syncthreads();
+    if (kt + 1 >= KT) break;
+    gload(R1);        // slice kt + 3
+    compute(1);       // slice kt + 1
+    sts(R0, 0);       // slice kt + 2
     __syncthreads();
   }
 
@@ -257,55 +274,68 @@ __global__ __launch_bounds__(256) void igemm_kernel(ConvGeom g, EpiArgs e)
   __syncthreads();
 
   // ---- epilogue ------------------------------------------------------------
-  // acc[t][s][r] = channel cb + 4*t + r of pixel m0 + wave_m*WM + 16*s + l16
+  // acc[t][s][r] = channel cb + 4*t + r of pixel m0 + wave_m*WM + 16*s + l16.
+  // Channel constants are fetched four channels (one MFMA tile row group) at a time to
+  // keep the register footprint of the epilogue below that of the main loop.
   const int cb = wave_n * WN + lgrp * (4 * TN);
-  int corr[4 * TN];
-  bn_t kk[4 * TN], ll[4 * TN];
+  const bool acc24 = g.K <= 256;  // |acc| <= K * 255 * 128 + 128 < 2^23
+  constexpr int QM = MODE == EPI_OUT32 ? EPI_RAW : MODE;
+  unsigned packed[TM][TN];
 #pragma unroll
-  for (int c = 0; c < 4 * TN; c++) {
-    const int n = n0 + cb + c;
-    int b = 0;
-    kk[c] = 0;
-    ll[c] = 0;
-    if (n < g.N) {
-      if (g.bias) b = (MODE == EPI_OUT32) ? ((const int *)g.bias)[n] : (int)g.bias[n];
-      if (MODE == EPI_BN) {
-        kk[c] = e.k[n];
-        ll[c] = e.lambda[n];
+  for (int t = 0; t < TN; t++) {
+    int corr[4];
+    bn_t kk[4], ll[4];
+    bool ks = true;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int n = n0 + cb + 4 * t + r;
+      int b = 0;
+      kk[r] = 0;
+      ll[r] = 0;
+      if (n < g.N) {
+        if (g.bias) b = (MODE == EPI_OUT32) ? ((const int *)g.bias)[n] : (int)g.bias[n];
+        if (MODE == EPI_BN) {
+          kk[r] = e.k[n];
+          ll[r] = e.lambda[n];
+        }
+      }
+      ks = ks && bn_k_small(kk[r]);
+      corr[r] = b + 128 * wsum[wave_n * WN + 16 * t + 4 * lgrp + r];
+    }
+    const bool k_small = __all(ks);  // wave-uniform precondition of the fast batch-norm form
+#pragma unroll
+    for (int s = 0; s < TM; s++) {
+      const int a0 = acc[t][s][0] + corr[0], a1 = acc[t][s][1] + corr[1];
+      const int a2 = acc[t][s][2] + corr[2], a3 = acc[t][s][3] + corr[3];
+      if constexpr (MODE == EPI_OUT32) {
+        const int m = m0 + wave_m * WM + 16 * s + l16;
+        if (m < g.M) {
+          int *o = (int *)g.out + (long long)m * g.N + n0 + cb + 4 * t;
+          const int v[4] = {a0, a1, a2, a3};
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (n0 + cb + 4 * t + r < g.N) o[r] = v[r];
+        }
+      } else {
+        packed[s][t] = acc24 ? requant4<QM, true>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift)
+                             : requant4<QM, false>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift);
       }
     }
-    corr[c] = b + 128 * wsum[wave_n * WN + 16 * (c >> 2) + 4 * lgrp + (c & 3)];
   }
+  if constexpr (MODE != EPI_OUT32) {
 #pragma unroll
-  for (int s = 0; s < TM; s++) {
-    const int m = m0 + wave_m * WM + 16 * s + l16;
-    if (m >= g.M) continue;
-    if constexpr (MODE == EPI_OUT32) {
-      int *o = (int *)g.out + (long long)m * g.N + n0 + cb;
-#pragma unroll
-      for (int c = 0; c < 4 * TN; c++)
-        if (n0 + cb + c < g.N) o[c] = acc[c >> 2][s][c & 3] + corr[c];
-    } else {
-      unsigned packed[TN];
-#pragma unroll
-      for (int t = 0; t < TN; t++) {
-        unsigned p = 0;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int c = 4 * t + r;
-          p |= (unsigned)requant<MODE == EPI_OUT32 ? EPI_RAW : MODE>(acc[t][s][r] + corr[c], kk[c], ll[c], e.mult, e.shift) << (8 * r);
-        }
-        packed[t] = p;
-      }
+    for (int s = 0; s < TM; s++) {
+      const int m = m0 + wave_m * WM + 16 * s + l16;
+      if (m >= g.M) continue;
       uint8_t *o = (uint8_t *)g.out + (long long)m * g.N + n0 + cb;
       if (g.vec_store && n0 + cb + 4 * TN <= g.N) {
-        if constexpr (TN == 4) *(uint4 *)o = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-        else if constexpr (TN == 2) *(uint2 *)o = make_uint2(packed[0], packed[1]);
-        else *(unsigned *)o = packed[0];
+        if constexpr (TN == 4) *(uint4 *)o = make_uint4(packed[s][0], packed[s][1], packed[s][2], packed[s][3]);
+        else if constexpr (TN == 2) *(uint2 *)o = make_uint2(packed[s][0], packed[s][1]);
+        else *(unsigned *)o = packed[s][0];
       } else {
 #pragma unroll
         for (int c = 0; c < 4 * TN; c++)
-          if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[c >> 2] >> (8 * (c & 3)));
+          if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[s][c >> 2] >> (8 * (c & 3)));
       }
     }
   }

@@ -70,20 +70,20 @@ bool epi_args(int mode, const bn_t *k, const bn_t *lambda, uint16_t out_mult, in
 
 // ---- implicit GEMM dispatch -------------------------------------------------
 
-template <int TN, int WM_, int WN_, int GATHER>
+template <int TN, int WM_, int WN_, int GATHER, int TM = 4>
 void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
-  constexpr int BM = 64 * WM_, BN = 16 * TN * WN_;
+  constexpr int BM = 16 * TM * WM_, BN = 16 * TN * WN_;
   const int tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   g.tiles_total = tiles_m * g.tiles_n;
   g.vec_store = (g.N % (4 * TN) == 0) && aligned(g.out, 4 * TN);
   dim3 grid(g.tiles_total), block(256);
   switch (mode) {
-    case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN>), grid, block, 0, s, g, e); break;
-    case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT>), grid, block, 0, s, g, e); break;
-    case EPI_RAW: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_RAW>), grid, block, 0, s, g, e); break;
-    default: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_OUT32>), grid, block, 0, s, g, e); break;
+    case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN, TM>), grid, block, 0, s, g, e); break;
+    case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT, TM>), grid, block, 0, s, g, e); break;
+    case EPI_RAW: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_RAW, TM>), grid, block, 0, s, g, e); break;
+    default: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_OUT32, TM>), grid, block, 0, s, g, e); break;
   }
 }
 
