@@ -24,9 +24,10 @@
 //     is one coalesced global load from the HWC input (GATHER_CHUNK16, needs
 //     Ci % 16 == 0), or a byte gather for any other geometry (GATHER_BYTES).
 #pragma once
-#include "requant.h"
+#include <type_traits>
 
-typedef int v4i __attribute__((ext_vector_type(4)));
+#include "memops.h"
+#include "requant.h"
 
 enum { GATHER_CHUNK16 = 0, GATHER_BYTES = 1 };
 enum { EPI_OUT32 = 3 };  // linear_out_32: int32 accumulators + int32 bias, no requantisation
@@ -43,6 +44,7 @@ struct ConvGeom {
   int pt, pl, sx, sy;
   long long in_img;    // bytes per input image
   int vec_store;       // output rows may be written with 4*TN-byte vector stores
+  int nt;              // write the output with non-temporal stores
   int tiles_n;         // number of channel tiles
   int tiles_total;     // tiles_m * tiles_n
 };
@@ -323,20 +325,26 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
     }
   }
   if constexpr (MODE != EPI_OUT32) {
+    // one copy of the store code per cache policy
+    auto put = [&](auto nt) {
+      constexpr bool NT = decltype(nt)::value;
 #pragma unroll
-    for (int s = 0; s < TM; s++) {
-      const int m = m0 + wave_m * WM + 16 * s + l16;
-      if (m >= g.M) continue;
-      uint8_t *o = (uint8_t *)g.out + (long long)m * g.N + n0 + cb;
-      if (g.vec_store && n0 + cb + 4 * TN <= g.N) {
-        if constexpr (TN == 4) *(uint4 *)o = make_uint4(packed[s][0], packed[s][1], packed[s][2], packed[s][3]);
-        else if constexpr (TN == 2) *(uint2 *)o = make_uint2(packed[s][0], packed[s][1]);
-        else *(unsigned *)o = packed[s][0];
-      } else {
+      for (int s = 0; s < TM; s++) {
+        const int m = m0 + wave_m * WM + 16 * s + l16;
+        if (m >= g.M) continue;
+        uint8_t *o = (uint8_t *)g.out + (long long)m * g.N + n0 + cb;
+        if (g.vec_store && n0 + cb + 4 * TN <= g.N) {
+          if constexpr (TN == 4) store16<NT>(o, (v4i){(int)packed[s][0], (int)packed[s][1 % TN], (int)packed[s][2 % TN], (int)packed[s][3 % TN]});
+          else if constexpr (TN == 2) store8<NT>(o, (v2i){(int)packed[s][0], (int)packed[s][1 % TN]});
+          else store4<NT>(o, (int)packed[s][0]);
+        } else {
 #pragma unroll
-        for (int c = 0; c < 4 * TN; c++)
-          if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[s][c >> 2] >> (8 * (c & 3)));
+          for (int c = 0; c < 4 * TN; c++)
+            if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[s][c >> 2] >> (8 * (c & 3)));
+        }
       }
-    }
+    };
+    if (g.nt) put(std::true_type{});
+    else put(std::false_type{});
   }
 }

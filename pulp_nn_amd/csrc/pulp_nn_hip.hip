@@ -78,6 +78,7 @@ void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   g.tiles_n = (g.N + BN - 1) / BN;
   g.tiles_total = tiles_m * g.tiles_n;
   g.vec_store = (g.N % (4 * TN) == 0) && aligned(g.out, 4 * TN);
+  g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
   dim3 grid(g.tiles_total), block(256);
   switch (mode) {
     case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN, TM>), grid, block, 0, s, g, e); break;
@@ -115,36 +116,49 @@ int num_cus()
   return n;
 }
 
-template <int TN, int KS>
+#ifndef PW_NW
+#define PW_NW 8  // waves per workgroup of the streaming kernel
+#endif
+#ifndef PW_TM
+#define PW_TM 2  // 16-pixel units per step
+#endif
+#ifndef PW_PER_CU
+#define PW_PER_CU 1
+#endif
+
+// Launches one instantiation; raises its dynamic-LDS limit above the default 64 KB as needed.
+template <auto KERN>
+void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t lds, hipStream_t s)
+{
+  static size_t limit = 65536;
+  if (lds > limit) {
+    (void)hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    limit = lds;
+  }
+  hipLaunchKernelGGL(KERN, grid, block, lds, s, g, e);
+}
+
+template <int TN, int NP, int KS>
 void launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
 {
-  constexpr int TM = 2;
-  dim3 block(256);
+  constexpr int TM = PW_TM, NW = PW_NW;
+  dim3 block(64 * NW);
   switch (mode) {
-    case EPI_BN:
-      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_BN, false, TM>), grid, block, lds, s, g, e);
-      break;
+    case EPI_BN: launch_pw<pw_stream_kernel<TN, KS, NP, EPI_BN, false, TM, NW>>(g, e, grid, block, lds, s); break;
     case EPI_MULT:
-      if (e.shift >= 16)
-        hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_MULT, true, TM>), grid, block, lds, s, g, e);
-      else
-        hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_MULT, false, TM>), grid, block, lds, s, g, e);
+      if (e.shift >= 16) launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, true, TM, NW>>(g, e, grid, block, lds, s);
+      else launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, false, TM, NW>>(g, e, grid, block, lds, s);
       break;
-    case EPI_RAW:
-      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_RAW, false, TM>), grid, block, lds, s, g, e);
-      break;
-    default:
-      hipLaunchKernelGGL((pw_stream_kernel<TN, KS, EPI_OUT32, false, TM>), grid, block, lds, s, g, e);
-      break;
+    default: launch_pw<pw_stream_kernel<TN, KS, NP, EPI_RAW, false, TM, NW>>(g, e, grid, block, lds, s); break;
   }
 }
 
-template <int TN>
+template <int TN, int NP>
 void launch_pw_stream_ks(int mode, int ks, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
 {
-  if (ks == 1) launch_pw_stream_mode<TN, 1>(mode, g, e, grid, lds, s);
-  else if (ks == 2) launch_pw_stream_mode<TN, 2>(mode, g, e, grid, lds, s);
-  else launch_pw_stream_mode<TN, 4>(mode, g, e, grid, lds, s);
+  if (ks == 1) launch_pw_stream_mode<TN, NP, 1>(mode, g, e, grid, lds, s);
+  else if (ks == 2) launch_pw_stream_mode<TN, NP, 2>(mode, g, e, grid, lds, s);
+  else launch_pw_stream_mode<TN, NP, 4>(mode, g, e, grid, lds, s);
 }
 
 // Weights-stationary streaming path: a GEMM whose rows are contiguous K-byte pixels,
@@ -161,7 +175,6 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   const int tn = N == 16 ? 1 : (N == 32 ? 2 : 4);
   const int np = N / (16 * tn);
   const int ks = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
-  constexpr int tm = 2;
   PwGeom g;
   g.in = in;
   g.w = w;
@@ -170,24 +183,22 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   g.M = (int)M;
   g.N = N;
   g.K = K;
-  const int lds = pw_lds_bytes(tn, ks, np, mode == EPI_BN);
-  if (lds > 65536) return false;
-  g.pgroups = (int)((M + 16 * tm - 1) / (16 * tm));
-  // Persistent grid: as many workgroups as stay resident, then trimmed so that every
-  // wave runs the same number of steps.
-  int per_cu = 163840 / lds;
-  if (per_cu > 2) per_cu = 2;  // measured: more resident workgroups do not stream faster
-  const int cap = per_cu * num_cus();
-  int blocks = (g.pgroups + 3) / 4;
-  if (blocks > cap) {
-    const int steps = (blocks + cap - 1) / cap;
-    blocks = (blocks + steps - 1) / steps;
-  }
+  const int lds = pw_lds_bytes(tn, ks, np, mode == EPI_BN, PW_NW, PW_TM);
+  if (lds > (160 * 1024 - 512) / PW_PER_CU) return false;  // 512: static LDS of the kernel
+  g.units = (int)((M + 15) / 16);
+  g.nt = M * N >= PULPNN_NT_BYTES;
+  // Persistent grid: one workgroup per CU (the weights are staged once per CU), fewer
+  // when there are not two 16-pixel units for every wave.
+  int blocks = PW_PER_CU * num_cus();
+  const int need = (g.units + 2 * PW_NW - 1) / (2 * PW_NW);
+  if (blocks > need) blocks = need;
   dim3 grid(blocks);
-  g.npass = np;
-  if (tn == 1) launch_pw_stream_ks<1>(mode, ks, g, e, grid, lds, s);
-  else if (tn == 2) launch_pw_stream_ks<2>(mode, ks, g, e, grid, lds, s);
-  else launch_pw_stream_ks<4>(mode, ks, g, e, grid, lds, s);
+  if (tn == 1) launch_pw_stream_ks<1, 1>(mode, ks, g, e, grid, lds, s);
+  else if (tn == 2) launch_pw_stream_ks<2, 1>(mode, ks, g, e, grid, lds, s);
+  else if (np == 1) launch_pw_stream_ks<4, 1>(mode, ks, g, e, grid, lds, s);
+  else if (np == 2) launch_pw_stream_ks<4, 2>(mode, ks, g, e, grid, lds, s);
+  else if (np == 3) launch_pw_stream_ks<4, 3>(mode, ks, g, e, grid, lds, s);
+  else launch_pw_stream_ks<4, 4>(mode, ks, g, e, grid, lds, s);
   return true;
 }
 

@@ -4,65 +4,92 @@
 // for 65 kop, far below the machine balance of ~625 op/B).
 //
 // The whole weight matrix sits in LDS in MFMA fragment order for the lifetime of
-// a (persistent) workgroup, together with the per-channel constants.  Every wave
-// streams its own pixels, 64 per step: the activation bytes go from HBM straight
-// into registers in the MFMA column-operand layout (lane = pixel l%16, 16-byte K
-// chunk l/16) and each byte is loaded by exactly one wave; the next step is
-// prefetched while the current one is multiplied against all channel groups,
-// requantised and stored.  There is no barrier after the weights are in place
-// and no im2col.
+// a (persistent) workgroup, one per CU, together with the per-channel constants.
+// Every wave owns a contiguous run of pixels and streams it 16*TM pixels per step:
+// the activation bytes go from HBM straight into registers in the MFMA
+// column-operand layout (lane = pixel l%16, 16-byte K chunk l/16), each byte is
+// loaded by exactly one wave, and the loads run two steps ahead of the arithmetic;
+// the first two steps are requested before the weights are staged, so that HBM is
+// busy while the workgroup sets up.  A step multiplies its pixels against every
+// channel group, requantises, gathers the channel groups of a pixel in a per-wave
+// LDS tile and writes whole pixel rows, 1 KB contiguous per store instruction.
+// There is no barrier after the set-up and no im2col.
+//
+// Everything the compiler has to count is fixed at compile time (loads and stores
+// per step, channel groups): loads and stores share one in-order counter on this
+// hardware, and only with a known number of stores behind a load can the wait for
+// that load leave the stores in flight.
 //
 // Arithmetic is that of igemm.h: activations as a ^ 0x80 with 128 * sum_k w
 // added back (by starting the accumulators at bias + 128 * sum_k w).
 #pragma once
+#include <type_traits>
+
 #include "igemm.h"
 #include "requant.h"
 
 struct PwGeom {
   const uint8_t *in;   // [M][K] pixels, K = Ci contiguous
   const int8_t *w;     // [N][K]
-  const int8_t *bias;  // int8 [N] (int32 for EPI_OUT32) or null
+  const int8_t *bias;  // int8 [N] or null
   void *out;           // [M][N]
   int M, N, K;
-  int npass;           // channel groups of 16*TN (N == npass * 16 * TN)
-  int pgroups;         // ceil(M / (16*TM)) pixel groups
+  int nt;              // write the output with non-temporal stores
+  int units;           // ceil(M / 16): 16-pixel units, dealt to the waves in equal contiguous runs
+#ifdef PW_TRACE
+  long long *dbg;
+#endif
 };
 
-// LDS bytes: weights, then k and lambda (bn_t), then corr (int) per padded channel, then a flag.
-static inline int pw_lds_bytes(int tn, int ks, int npass, bool bn)
+// LDS bytes: weights, then k and lambda (bn_t), then corr (int) per channel; with more
+// than one channel group per pixel, a private output tile per wave of 16*tm rows of
+// N + 16 bytes.
+__host__ __device__ static inline int pw_lds_fixed(int tn, int ks, int np, bool bn)
 {
-  return npass * 16 * tn * (ks * 64 + 4 + (bn ? 2 * (int)sizeof(bn_t) : 0)) + 16;
+  return np * 16 * tn * (ks * 64 + 4 + (bn ? 2 * (int)sizeof(bn_t) : 0));
+}
+static inline int pw_lds_bytes(int tn, int ks, int np, bool bn, int nw, int tm)
+{
+  const int n = np * 16 * tn;
+  return pw_lds_fixed(tn, ks, np, bn) + (np > 1 ? nw * 16 * tm * (n + 16) : 0);
 }
 
-template <int TN, int KS, int MODE, bool WIDE, int TM>
-__global__ __launch_bounds__(256, TM == 2 ? 4 : 2) void pw_stream_kernel(PwGeom g, EpiArgs e)
+// N == NP * 16 * TN: every lane owns 4*TN real channels of each of the NP channel groups.
+template <int TN, int KS, int NP, int MODE, bool WIDE, int TM, int NW>
+__global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwGeom g, EpiArgs e)
 {
-  // N == NP * 16 * TN: every lane owns 4*TN real channels
-  constexpr int PX = 16 * TM;  // pixels per step
-  constexpr int CG = 16 * TN;  // channels per pass
+  constexpr int BS = 64 * NW;      // threads per workgroup
+  constexpr int PX = 16 * TM;      // pixels per step
+  constexpr int CG = 16 * TN;      // channels per group
+  constexpr int N = NP * CG;       // output channels
+  constexpr bool XP = NP > 1;      // gather the groups of a pixel in LDS before storing
+  constexpr int OROW = N + 16;     // row pitch of the output tile: the 16 bytes of padding spread
+                                   // the pieces that 16 pixel lanes write at equal channel
+                                   // offsets over all banks
   extern __shared__ __attribute__((aligned(16))) unsigned char pw_lds[];
-  const int npad = g.npass * CG;
   int8_t *Wl = (int8_t *)pw_lds;
-  bn_t *kl = (bn_t *)(pw_lds + npad * KS * 64);
-  bn_t *ll_ = kl + ((MODE == EPI_BN) ? npad : 0);
-  int *corr_l = (int *)(ll_ + ((MODE == EPI_BN) ? npad : 0));
-  int *flag_l = corr_l + npad;
+  bn_t *kl = (bn_t *)(pw_lds + N * KS * 64);
+  bn_t *ll_ = kl + ((MODE == EPI_BN) ? N : 0);
+  int *corr_l = (int *)(ll_ + ((MODE == EPI_BN) ? N : 0));
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
   const int l16 = lane & 15, lgrp = lane >> 4;
+  unsigned char *ob = pw_lds + pw_lds_fixed(TN, KS, NP, MODE == EPI_BN) + wave * (PX * OROW);
 
-  // ---- first pixels on their way before anything else ---------------------------
-  const int nwaves = gridDim.x * 4;
-  int pg = blockIdx.x * 4 + wave;
+  // ---- this wave's share of the pixels ---------------------------------------------------
+  // This wave's pixels: an equal share of the 16-pixel units, contiguous in memory.
+  const int nwaves = gridDim.x * NW, gw = blockIdx.x * NW + wave;
+  const int px_end = min((int)((long long)g.units * (gw + 1) / nwaves) * 16, g.M);
+  int px = (int)((long long)g.units * gw / nwaves) * 16;
   // Unconditional loads from clamped addresses (no per-lane branches, so that all
   // loads of a step are issued back to back and nothing waits on them here):
-  // pixels past the end re-read the last pixel (their results are never stored) and
-  // K chunks past the end re-read chunk 0 (their weights are zero).
-  auto load_a = [&](v4i (&a)[TM][KS], int pgi) {
+  // pixels past the end of the run re-read its last pixel and K chunks past the end
+  // re-read chunk 0 (their weights are zero).
+  auto load_a = [&](v4i (&a)[TM][KS], int p0) {
 #pragma unroll
     for (int s = 0; s < TM; s++) {
-      const int m = min(pgi * PX + 16 * s + l16, g.M - 1);
+      const int m = max(min(p0 + 16 * s + l16, px_end - 1), 0);
       const uint8_t *row = g.in + (long long)m * g.K;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
@@ -71,71 +98,99 @@ __global__ __launch_bounds__(256, TM == 2 ? 4 : 2) void pw_stream_kernel(PwGeom 
       }
     }
   };
-  v4i cur[TM][KS], nxt[TM][KS];
-  load_a(cur, min(pg, g.pgroups - 1));
+  v4i b0[TM][KS], b1[TM][KS], b2[TM][KS];
+#ifdef PW_TRACE
+  int trc = 0;
+  auto TR = [&]() { if (lane == 0 && trc < 12) g.dbg[gw * 12 + trc] = wall_clock64(); trc++; };
+  TR();
+#else
+#define TR()
+#endif
 
   // ---- weights and per-channel constants -> LDS -----------------------------------
-  for (int n = tid; n < npad; n += 256) corr_l[n] = 0;
-  if (tid == 0) *flag_l = 1;
-  __syncthreads();
-  {
-    const int rows = npad * KS;  // 64-byte rows
-    bool small = true;
-    // batches of 8 chunks per thread so that 8 loads are in flight before the first LDS write
-    for (int q0 = tid; q0 < rows * 4; q0 += 256 * 8) {
-      v4i v[8];
-      int nn[8];
+  // All global loads of the set-up are issued before the first of them is consumed.
+  constexpr int CHUNKS = N * KS * 4;             // 16-byte chunks of the padded weight matrix
+  constexpr int CH = (CHUNKS + BS - 1) / BS;     // per thread
+  constexpr int NC = (N + BS - 1) / BS;          // channels per thread
+  v4i wv[CH];
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        const int q = q0 + 256 * u;
-        const int R = q >> 2, c = q & 3;
-        const int i = R & 15, t = (R >> 4) % TN, ks = (R / CG) % KS, p = R / (CG * KS);
-        nn[u] = p * CG + (i >> 2) * (4 * TN) + 4 * t + (i & 3);
-        const int k = ks * 64 + 16 * c;
-        v[u] = (v4i){0, 0, 0, 0};
-        if (q < rows * 4 && nn[u] < g.N && k < g.K) v[u] = *(const v4i *)(g.w + (long long)nn[u] * g.K + k);
-      }
+  for (int u = 0; u < CH; u++) {
+    // LDS row R = ((p*KS + ks)*TN + t)*16 + i holds channel p*CG + (i/4)*4*TN + 4*t + i%4
+    const int q = tid + BS * u, R = q >> 2, c = q & 3;
+    const int i = R & 15, t = (R >> 4) % TN, ks = (R / CG) % KS, p = R / (CG * KS);
+    const int n = p * CG + (i >> 2) * (4 * TN) + 4 * t + (i & 3);
+    const int k = ks * 64 + 16 * c;
+    const bool ok = q < CHUNKS && k < g.K;
+    wv[u] = *(const v4i *)(g.w + (ok ? (long long)n * g.K + k : 0));
+  }
+  int bv[NC];
+  bn_t kv[NC], lv[NC];
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        const int q = q0 + 256 * u;
-        if (q >= rows * 4) break;  // uniform across the wave: rows * 4 is a multiple of 64
-        const int R = q >> 2, c = q & 3;
-        *(v4i *)&Wl[lds_off(R, c)] = v[u];
-        int part = __builtin_amdgcn_sdot4(v[u].x, 0x01010101, 0, false);
-        part = __builtin_amdgcn_sdot4(v[u].y, 0x01010101, part, false);
-        part = __builtin_amdgcn_sdot4(v[u].z, 0x01010101, part, false);
-        part = __builtin_amdgcn_sdot4(v[u].w, 0x01010101, part, false);
-        part += __shfl_xor(part, 1);
-        part += __shfl_xor(part, 2);
-        if (c == 0) atomicAdd(&corr_l[nn[u]], 128 * part);
+  for (int u = 0; u < NC; u++) {
+    const int n = min(tid + BS * u, N - 1);
+    bv[u] = g.bias ? (int)g.bias[n] : 0;
+    if constexpr (MODE == EPI_BN) {
+      kv[u] = e.k[n];
+      lv[u] = e.lambda[n];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < CH; u++) {
+    const int q = tid + BS * u, R = q >> 2, c = q & 3;
+    const int k = ((R / CG) % KS) * 64 + 16 * c;
+    if (q < CHUNKS) *(v4i *)&Wl[lds_off(R, c)] = (k < g.K) ? wv[u] : (v4i){0, 0, 0, 0};
+  }
+  // The first two steps' pixels are requested only now: the CU's memory pipeline serves
+  // requests in order, and the (few, mostly L2-resident) set-up loads are not to queue
+  // behind 64 KB of pixels from HBM.
+  load_a(b0, px);
+  load_a(b1, px + PX);
+  TR();
+  bool small = true;
+#pragma unroll
+  for (int u = 0; u < NC; u++) {
+    const int n = tid + BS * u;
+    if (n < N) {
+      corr_l[n] = bv[u];
+      if constexpr (MODE == EPI_BN) {
+        kl[n] = kv[u];
+        ll_[n] = lv[u];
+        small = small && bn_k_small(kv[u]);
       }
     }
-    for (int n = tid; n < npad; n += 256) {
-      int b = 0;
-      if (n < g.N && g.bias) b = (MODE == EPI_OUT32) ? ((const int *)g.bias)[n] : (int)g.bias[n];
-      if (b) atomicAdd(&corr_l[n], b);
-      if (MODE == EPI_BN) {
-        const bn_t kv = n < g.N ? e.k[n] : 0;
-        kl[n] = kv;
-        ll_[n] = n < g.N ? e.lambda[n] : 0;
-        small = small && bn_k_small(kv);
-      }
+  }
+  const bool k_small = __syncthreads_and(small);
+  TR();
+  // corr = bias + 128 * sum_k w: the row sums of a weight tile are its product with a
+  // matrix of ones; each tile has one owner wave and each channel one owner lane.
+  for (int tile = wave; tile < NP * TN; tile += NW) {
+    const int p = tile / TN, t = tile % TN;
+    v4i acc = {0, 0, 0, 0};
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const v4i wf = *(const v4i *)&Wl[lds_off(((p * KS + ks) * TN + t) * 16 + l16, lgrp)];
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf, ones, acc, 0, 0, 0);
     }
-    if (!small) *flag_l = 0;
+    if (l16 == 0) {
+      v4i *c4 = (v4i *)&corr_l[p * CG + lgrp * (4 * TN) + 4 * t];
+      *c4 = *c4 + acc * 128;
+    }
   }
   __syncthreads();
-  const bool k_small = *flag_l != 0;
+  TR();
 
   // ---- stream pixels ------------------------------------------------------------------
-  // One step: 64 pixels against every channel group.
-  auto process = [&](v4i (&a)[TM][KS], int pgi) {
+  // One step: 16 * TM pixels against every channel group.
+  auto process = [&](v4i (&a)[TM][KS], int p0, auto nt) {
+    constexpr bool NT = decltype(nt)::value;
 #pragma unroll
     for (int s = 0; s < TM; s++)
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) a[s][ks] ^= (int)0x80808080;
 
 #pragma unroll 1
-    for (int p = 0; p < g.npass; p++) {
+    for (int p = 0; p < NP; p++) {
       const int cb = p * CG + lgrp * (4 * TN);  // first of this lane's 4*TN channels
       v4i acc[TN][TM];
 #pragma unroll
@@ -155,55 +210,74 @@ __global__ __launch_bounds__(256, TM == 2 ? 4 : 2) void pw_stream_kernel(PwGeom 
           }
         }
 
-      if constexpr (MODE == EPI_OUT32) {
+      bn_t kk[4 * TN], lam[4 * TN];
+      if constexpr (MODE == EPI_BN) {
 #pragma unroll
-        for (int s = 0; s < TM; s++) {
-          const int m = pgi * PX + 16 * s + l16;
-          if (m >= g.M) continue;
-          int *o = (int *)g.out + (long long)m * g.N + cb;
-#pragma unroll
-          for (int c = 0; c < 4 * TN; c++)
-            if (cb + c < g.N) o[c] = acc[c >> 2][s][c & 3];
+        for (int c = 0; c < 4 * TN; c++) {
+          kk[c] = kl[cb + c];
+          lam[c] = ll_[cb + c];
         }
-      } else {
-        bn_t kk[4 * TN], lam[4 * TN];
-        if constexpr (MODE == EPI_BN) {
+      }
 #pragma unroll
-          for (int c = 0; c < 4 * TN; c++) {
-            kk[c] = kl[cb + c];
-            lam[c] = ll_[cb + c];
-          }
-        }
+      for (int s = 0; s < TM; s++) {
+        unsigned packed[TN];
 #pragma unroll
-        for (int s = 0; s < TM; s++) {
-          const int m = pgi * PX + 16 * s + l16;
-          unsigned packed[TN];
-#pragma unroll
-          for (int t = 0; t < TN; t++)
-            packed[t] = requant4<MODE, true, WIDE>(acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3], &kk[4 * t],
-                                                   &lam[4 * t], k_small, e.mult, e.shift);
-          {
-            // Every lane stores, without a branch: lanes past the last pixel hold the
-            // results of the last pixel (their loads were clamped to it) and rewrite them.
-            uint8_t *o = (uint8_t *)g.out + (long long)min(m, g.M - 1) * g.N + cb;
-            if constexpr (TN == 4) *(uint4 *)o = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-            else if constexpr (TN == 2) *(uint2 *)o = make_uint2(packed[0], packed[1]);
-            else *(unsigned *)o = packed[0];
-          }
+        for (int t = 0; t < TN; t++)
+          packed[t] = requant4<MODE, true, WIDE>(acc[t][s][0], acc[t][s][1], acc[t][s][2], acc[t][s][3], &kk[4 * t],
+                                                 &lam[4 * t], k_small, e.mult, e.shift);
+        if constexpr (XP) {
+          static_assert(!XP || TN == 4, "output tile rows are written 16 bytes at a time");
+          *(v4i *)(ob + (16 * s + l16) * OROW + cb) = (v4i){(int)packed[0], (int)packed[1 % TN], (int)packed[2 % TN], (int)packed[3 % TN]};
+        } else {
+          // Every lane stores, without a branch: lanes past the last pixel of the run hold
+          // the results of that pixel (their loads were clamped to it) and rewrite them.
+          const int m = min(p0 + 16 * s + l16, px_end - 1);
+          uint8_t *o = (uint8_t *)g.out + (long long)m * N + cb;
+          if constexpr (TN == 4) store16<NT>(o, (v4i){(int)packed[0], (int)packed[1 % TN], (int)packed[2 % TN], (int)packed[3 % TN]});
+          else if constexpr (TN == 2) store8<NT>(o, (v2i){(int)packed[0], (int)packed[1 % TN]});
+          else store4<NT>(o, (int)packed[0]);
         }
       }
     }
+    if constexpr (XP) {
+      // The tile in memory order: piece idx = r*64 + lane is bytes [16*idx, 16*idx + 16) of the
+      // step's PX * N contiguous output bytes.  Rows past the end of the run are redirected
+      // to its last row (same bytes to the same address): no branch, fixed store count.
+      constexpr int CPR = N / 16, NR = PX * N / 1024;
+      const int last = px_end - 1 - p0;
+      v4i v[NR];
+      long long go[NR];
+#pragma unroll
+      for (int r = 0; r < NR; r++) {
+        const int idx = r * 64 + lane, row = min(idx / CPR, last), col = (idx % CPR) * 16;
+        v[r] = *(const v4i *)(ob + row * OROW + col);
+        go[r] = (long long)(p0 + row) * N + col;
+      }
+#pragma unroll
+      for (int r = 0; r < NR; r++) store16<NT>((uint8_t *)g.out + go[r], v[r]);
+    }
   };
 
-  // One step per iteration: the loads of the next step are issued first, unconditionally
-  // (clamped to the last group) and into registers nothing else touches, so that the only
-  // wait on them is the register hand-over at the bottom of the loop.
-  for (; pg < g.pgroups; pg += nwaves) {
-    load_a(nxt, min(pg + nwaves, g.pgroups - 1));
-    process(cur, pg);
+  // Three register sets: the loads of step i+2 are issued, unconditionally (clamped to the
+  // end of the run), before step i is computed.  The sets are handed down by register
+  // moves in a single-copy loop body: the compiler derives how long a load may stay in
+  // flight from the instructions issued behind it, and an unrolled rotation makes it merge
+  // three different histories at the loop header into a wait for everything.
+  auto stream = [&](auto nt) {
+    for (; px < px_end; px += PX) {
+      load_a(b2, px + 2 * PX);
+      process(b0, px, nt);
+      TR();
 #pragma unroll
-    for (int s = 0; s < TM; s++)
+      for (int s = 0; s < TM; s++)
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) cur[s][ks] = nxt[s][ks];
-  }
+        for (int ks = 0; ks < KS; ks++) {
+          b0[s][ks] = b1[s][ks];
+          b1[s][ks] = b2[s][ks];
+        }
+    }
+  };
+  // the store policy is fixed per launch: one copy of the loop for each, no branch per store
+  if (g.nt) stream(std::true_type{});
+  else stream(std::false_type{});
 }
