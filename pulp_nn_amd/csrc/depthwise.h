@@ -22,9 +22,9 @@
 //      "4 pixels of my channel" into "4 channels of one pixel", so that 16
 //      quads write 64 contiguous bytes of an HWC pixel.
 #pragma once
+#include "memops.h"
 #include "requant.h"
 
-typedef int v4i __attribute__((ext_vector_type(4)));
 
 struct DwGeom {
   const uint8_t *in;
@@ -45,6 +45,7 @@ struct DwGeom {
   int inc_dw, inc_row, inc_c;
   int in_align4;  // input pointer and W are multiples of 4: aligned dword loads are safe
   int out_vec4;   // output pointer and CH are multiples of 4: dword stores are safe
+  int nt;         // write the output with non-temporal stores
 };
 
 #define DW_CG 64  // channels per workgroup (one per lane)
@@ -237,7 +238,7 @@ struct DwColumn {
   int store, nbytes;
 };
 
-template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ>
+template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ, bool NT = false>
 __device__ __forceinline__ void dw3x3_column(DwColumn c)
 {
   constexpr int O0 = 4 - PL;
@@ -261,7 +262,7 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
     unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], c.k, c.lambda, c.mult, c.shift);
     packed = quad_transpose4x4_perm(packed, c.sel1, c.sel2);
     if constexpr (FULL) {
-      *(unsigned *)c.o = packed;
+      store4<NT>(c.o, (int)packed);
     } else {
       if (c.store == 0) {
         *(unsigned *)c.o = packed;
@@ -451,7 +452,11 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
     col.store = (4 * xg + (lane & 3) >= g.Wo) ? 2 : ((g.out_vec4 && c0 + cq + 3 < g.CH) ? 0 : 1);
     col.nbytes = min(4, g.CH - c0 - cq);
     const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
-    if (fastq) {
+    if (FULL && fastq && g.nt) {
+      // one more copy of the common case for the streaming store policy
+      if (edge) dw3x3_column<S, PL, MODE, FULL, true, true, FULL>(col);
+      else dw3x3_column<S, PL, MODE, FULL, false, true, FULL>(col);
+    } else if (fastq) {
       if (edge) dw3x3_column<S, PL, MODE, FULL, true, true>(col);
       else dw3x3_column<S, PL, MODE, FULL, false, true>(col);
     } else {
@@ -548,6 +553,88 @@ __global__ __launch_bounds__(256) void hwc_to_chw_kernel(const uint8_t *in, uint
       if (c >= C) continue;
       for (int x = tx; x < pad_t * W; x += 64) dst[(long long)c * Hp * W + x] = 0;
       for (int x = tx; x < pad_b * W; x += 64) dst[((long long)c * Hp + pad_t + H) * W + x] = 0;
+    }
+  }
+}
+
+// 4x4 byte transpose inside one lane: r[i] = bytes of pixel i (4 channels) ->
+// t[j] = bytes of channel j (4 pixels).
+__device__ __forceinline__ void transpose4x4_bytes(const unsigned (&r)[4], unsigned (&t)[4])
+{
+  // __builtin_amdgcn_perm(hi, lo, sel): selector 0-3 picks bytes of lo, 4-7 bytes of hi
+  const unsigned a0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400);  // p0c0 p1c0 p0c1 p1c1
+  const unsigned a1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602);  // p0c2 p1c2 p0c3 p1c3
+  const unsigned b0 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400);  // p2c0 p3c0 p2c1 p3c1
+  const unsigned b1 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602);
+  t[0] = __builtin_amdgcn_perm(b0, a0, 0x05040100);
+  t[1] = __builtin_amdgcn_perm(b0, a0, 0x07060302);
+  t[2] = __builtin_amdgcn_perm(b1, a1, 0x05040100);
+  t[3] = __builtin_amdgcn_perm(b1, a1, 0x07060302);
+}
+
+// Fast HWC -> CHW for C % 16 == 0, H*W % 4 == 0 and 16-byte aligned maps: a tile of
+// 256 pixels x 64 channels goes through LDS; reads are 16 bytes per lane (64 contiguous
+// bytes per pixel), writes are one dword of 4 pixels per lane, 256 contiguous bytes per
+// channel and store instruction.
+template <bool NT>
+__global__ __launch_bounds__(256) void hwc_to_chw_fast_kernel(const uint8_t *in, uint8_t *out, int H, int W, int C,
+                                                              int pad_t, int pad_b, int tiles_p, int tiles_c)
+{
+  constexpr int P = 80;  // LDS row pitch in bytes (16-byte aligned rows)
+  __shared__ __attribute__((aligned(16))) uint8_t tile[256 * P];
+  int id = blockIdx.x;
+  const int tc = id % tiles_c;
+  id /= tiles_c;
+  const int tp = id % tiles_p;
+  const int b = id / tiles_p;
+  const int HW = H * W;
+  const int Hp = pad_t + H + pad_b;
+  const uint8_t *src = in + (long long)b * HW * C;
+  uint8_t *dst = out + (long long)b * C * Hp * W;
+  const int p0 = tp * 256, c0 = tc * 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  {
+    const int chunk = tid & 3, c = c0 + 16 * chunk;
+    v4i v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int p = min(p0 + (tid >> 2) + 64 * i, HW - 1);
+      v[i] = *(const v4i *)(src + (long long)p * C + min(c, C - 16));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) *(v4i *)&tile[((tid >> 2) + 64 * i) * P + 16 * chunk] = v[i];
+  }
+  __syncthreads();
+  const int cw = c0 + 16 * wave;  // this wave's 16 channels
+  const int p = p0 + 4 * lane;    // this lane's 4 pixels
+  if (cw < C && p < HW) {
+    unsigned rows[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const v4i r = *(const v4i *)&tile[(4 * lane + i) * P + 16 * wave];
+      rows[i][0] = (unsigned)r.x;
+      rows[i][1] = (unsigned)r.y;
+      rows[i][2] = (unsigned)r.z;
+      rows[i][3] = (unsigned)r.w;
+    }
+    uint8_t *o = dst + ((long long)cw * Hp + pad_t) * W + p;
+    const long long plane = (long long)Hp * W;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+      const unsigned r[4] = {rows[0][d], rows[1][d], rows[2][d], rows[3][d]};
+      unsigned t[4];
+      transpose4x4_bytes(r, t);
+#pragma unroll
+      for (int j = 0; j < 4; j++) store4<NT>(o + (4 * d + j) * plane, (int)t[j]);
+    }
+  }
+  // zero rows
+  if (tp == 0 && (pad_t | pad_b)) {
+    for (int i = wave; i < 64; i += 4) {
+      const int c = c0 + i;
+      if (c >= C) continue;
+      for (int x = lane; x < pad_t * W; x += 64) dst[(long long)c * Hp * W + x] = 0;
+      for (int x = lane; x < pad_b * W; x += 64) dst[((long long)c * Hp + pad_t + H) * W + x] = 0;
     }
   }
 }

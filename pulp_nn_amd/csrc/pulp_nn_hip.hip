@@ -352,6 +352,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.inc_c = carry / g.NR;
   g.in_align4 = aligned(in, 4) && (W % 4 == 0);
   g.out_vec4 = aligned(out, 4) && (CH % 4 == 0);
+  g.nt = (long long)g.B * Ho * Wo * CH >= PULPNN_NT_BYTES;
   const size_t lds = (size_t)DW_CG * g.CSD * 4;
   dim3 grid(g.total), block(256);
 #define DW_LAUNCH(KERNEL)                                                                   \
@@ -478,6 +479,21 @@ void pulp_nn_hip_hwc_to_chw(const unsigned char *in_hwc, unsigned char *out_chw,
 {
   REQUIRE(in_hwc && out_chw, PULP_NN_HIP_ERR_ARGUMENT, "null pointer");
   REQUIRE(dim_x && dim_y && ch, PULP_NN_HIP_ERR_ARGUMENT, "zero dimension");
+  const unsigned hw = dim_x * dim_y, plane = (pad_top + dim_y + pad_bottom) * dim_x;
+  if (ch % 16 == 0 && hw % 4 == 0 && plane % 4 == 0 && (pad_top * dim_x) % 4 == 0 && aligned(in_hwc, 16) &&
+      aligned(out_chw, 4)) {
+    const int tiles_p = (int)((hw + 255) / 256), tiles_c = (int)((ch + 63) / 64);
+    const long long total = (long long)g_batch * tiles_p * tiles_c;
+    REQUIRE(total <= 0x7fffffffLL, PULP_NN_HIP_ERR_ARGUMENT, "batch too large");
+    if ((long long)g_batch * hw * ch >= PULPNN_NT_BYTES)
+      hipLaunchKernelGGL(hwc_to_chw_fast_kernel<true>, dim3((unsigned)total), dim3(256), 0, g_stream, in_hwc, out_chw,
+                         (int)dim_y, (int)dim_x, (int)ch, (int)pad_top, (int)pad_bottom, tiles_p, tiles_c);
+    else
+      hipLaunchKernelGGL(hwc_to_chw_fast_kernel<false>, dim3((unsigned)total), dim3(256), 0, g_stream, in_hwc, out_chw,
+                         (int)dim_y, (int)dim_x, (int)ch, (int)pad_top, (int)pad_bottom, tiles_p, tiles_c);
+    check_launch(__func__);
+    return;
+  }
   const int tiles_p = (int)((dim_x * dim_y + 63) / 64), tiles_c = (int)((ch + 63) / 64);
   const long long total = (long long)g_batch * tiles_p * tiles_c;
   REQUIRE(total <= 0x7fffffffLL, PULP_NN_HIP_ERR_ARGUMENT, "batch too large");
@@ -563,7 +579,15 @@ void pulp_nn_maxpool(uint8_t *Im_in, uint8_t *Im_out, uint16_t dim_im_in_x, uint
   // i_x >= 1 with i_x*stride_x - padding_l < i_x (pulp_nn_maxpool.c:58-94).
   REQUIRE(padding_l == 0 || (int)stride_x - 1 >= (int)padding_l, PULP_NN_HIP_ERR_UNSUPPORTED,
           "left padding this large makes the reference's in-place x pass order dependent");
-  hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((g.total + 255) / 256)), dim3(256), 0, g_stream, g);
+  if (ch_im_in % 16 == 0 && aligned(Im_in, 16) && aligned(Im_out, 16)) {
+    g.cgroups = ch_im_in / 16;
+    g.total = (long long)g.B * g.Ho * g.Wo * g.cgroups;
+    const dim3 grid((unsigned)((g.total + 255) / 256));
+    if (g.total * 16 >= PULPNN_NT_BYTES) hipLaunchKernelGGL(maxpool16_kernel<true>, grid, dim3(256), 0, g_stream, g);
+    else hipLaunchKernelGGL(maxpool16_kernel<false>, grid, dim3(256), 0, g_stream, g);
+  } else {
+    hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((g.total + 255) / 256)), dim3(256), 0, g_stream, g);
+  }
   check_launch(__func__);
 }
 

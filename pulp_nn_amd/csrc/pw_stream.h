@@ -36,9 +36,6 @@ struct PwGeom {
   int M, N, K;
   int nt;              // write the output with non-temporal stores
   int units;           // ceil(M / 16): 16-pixel units, dealt to the waves in equal contiguous runs
-#ifdef PW_TRACE
-  long long *dbg;
-#endif
 };
 
 // LDS bytes: weights, then k and lambda (bn_t), then corr (int) per channel; with more
@@ -99,13 +96,6 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
     }
   };
   v4i b0[TM][KS], b1[TM][KS], b2[TM][KS];
-#ifdef PW_TRACE
-  int trc = 0;
-  auto TR = [&]() { if (lane == 0 && trc < 12) g.dbg[gw * 12 + trc] = wall_clock64(); trc++; };
-  TR();
-#else
-#define TR()
-#endif
 
   // ---- weights and per-channel constants -> LDS -----------------------------------
   // All global loads of the set-up are issued before the first of them is consumed.
@@ -145,7 +135,6 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
   // behind 64 KB of pixels from HBM.
   load_a(b0, px);
   load_a(b1, px + PX);
-  TR();
   bool small = true;
 #pragma unroll
   for (int u = 0; u < NC; u++) {
@@ -160,7 +149,6 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
     }
   }
   const bool k_small = __syncthreads_and(small);
-  TR();
   // corr = bias + 128 * sum_k w: the row sums of a weight tile are its product with a
   // matrix of ones; each tile has one owner wave and each channel one owner lane.
   for (int tile = wave; tile < NP * TN; tile += NW) {
@@ -178,7 +166,6 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
     }
   }
   __syncthreads();
-  TR();
 
   // ---- stream pixels ------------------------------------------------------------------
   // One step: 16 * TM pixels against every channel group.
@@ -267,7 +254,6 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
     for (; px < px_end; px += PX) {
       load_a(b2, px + 2 * PX);
       process(b0, px, nt);
-      TR();
 #pragma unroll
       for (int s = 0; s < TM; s++)
 #pragma unroll
