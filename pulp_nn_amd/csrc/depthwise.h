@@ -286,17 +286,25 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
     for (int j = 0; j < 4; j++) Q[j] = c.corr;
     taps(span, 1, P);
     taps(span, 0, Q);
-    for (int r = 0; r < c.rows; r++) {
+    // Three accumulator sets take the roles (finishing, middle, starting) in turn; the
+    // loop is unrolled by three so that the hand-over costs no register moves.
+    int R[4];
+    auto step = [&](int (&fin)[4], int (&mid)[4], int (&beg)[4]) {
       read_row(span);
-      taps(span, 2, P);
-      emit(P);
+      taps(span, 2, fin);
+      emit(fin);
+      taps(span, 1, mid);
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        P[j] = Q[j];
-        Q[j] = c.corr;
-      }
-      taps(span, 1, P);
-      taps(span, 0, Q);
+      for (int j = 0; j < 4; j++) beg[j] = c.corr;
+      taps(span, 0, beg);
+    };
+    for (int r = 0; c.rows > 0;) {
+      step(P, Q, R);
+      if (++r >= c.rows) break;
+      step(Q, R, P);
+      if (++r >= c.rows) break;
+      step(R, P, Q);
+      if (++r >= c.rows) break;
     }
   } else {
     // Q: next output row so far (K0 row done)
