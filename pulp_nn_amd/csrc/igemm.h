@@ -23,13 +23,20 @@
 //   * The im2col gather is never materialised: each 16-byte chunk of a K slice
 //     is one coalesced global load from the HWC input (GATHER_CHUNK16, needs
 //     Ci % 16 == 0), or a byte gather for any other geometry (GATHER_BYTES).
+//     With Ci % 64 == 0 (GATHER_UNIFORM) a whole K slice lies inside one filter tap, so
+//     the tap walk is scalar work shared by the wave, and the loads are buffer loads whose
+//     hardware range check supplies the zeros: a pixel's offset is fixed for the whole
+//     kernel, the tap adds a scalar offset, and an out-of-image tap (one bit per tap and
+//     pixel, computed once) ORs the offset to 0xffffffff, which the range check turns
+//     into a load of zeros.  Per K slice that is two VALU instructions per 16-byte chunk
+//     of activations and none per chunk of weights.
 #pragma once
 #include <type_traits>
 
 #include "memops.h"
 #include "requant.h"
 
-enum { GATHER_CHUNK16 = 0, GATHER_BYTES = 1 };
+enum { GATHER_CHUNK16 = 0, GATHER_BYTES = 1, GATHER_UNIFORM = 2 };
 enum { EPI_OUT32 = 3 };  // linear_out_32: int32 accumulators + int32 bias, no requantisation
 
 struct ConvGeom {
@@ -51,7 +58,7 @@ struct ConvGeom {
 
 #define IGEMM_BK 64
 #ifndef IGEMM_MINB
-#define IGEMM_MINB 2  // workgroups per CU the register budget is sized for
+#define IGEMM_MINB 3  // workgroups per CU the register budget is sized for
 #endif
 
 // Tile index of this workgroup.  Workgroups are dealt round-robin to the 8
@@ -70,14 +77,18 @@ __device__ __forceinline__ int lds_off(int row, int chunk)
 }
 
 template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4>
-__global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiArgs e)
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, WAVES_M * WAVES_N > 4 ? 1 : (GATHER == GATHER_BYTES ? 2 : IGEMM_MINB))
+void igemm_kernel(ConvGeom g, EpiArgs e)
 {
   constexpr int WM = 16 * TM, WN = 16 * TN;
   constexpr int BM = WM * WAVES_M, BN = WN * WAVES_N;
-  constexpr int RA = BM / 64;                    // activation chunks per thread per K slice
-  constexpr int RW = (BN * 4 + 255) / 256;       // weight chunks per thread per K slice
-  static_assert(WAVES_M * WAVES_N == 4, "256 threads");
+  constexpr int NTH = 64 * WAVES_M * WAVES_N;    // threads per workgroup
+  constexpr int RPP = NTH / 4;                   // tile rows staged per pass (4 threads per 64-byte row)
+  constexpr int RA = BM / RPP;                   // activation chunks per thread per K slice
+  constexpr int RW = (BN * 4 + NTH - 1) / NTH;   // weight chunks per thread per K slice
+  static_assert(BM % RPP == 0, "pixel tile is a whole number of staging passes");
 
+  constexpr bool UNI = GATHER == GATHER_UNIFORM;  // scalar tap walk and buffer loads
   __shared__ __attribute__((aligned(16))) uint8_t As[2][BM * IGEMM_BK];
   __shared__ __attribute__((aligned(16))) int8_t Ws[2][BN * IGEMM_BK];
   __shared__ int wsum[BN];
@@ -96,7 +107,7 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
   long long abase[RA];
 #pragma unroll
   for (int i = 0; i < RA; i++) {
-    const int m = m0 + (tid >> 2) + 64 * i;
+    const int m = m0 + (tid >> 2) + RPP * i;
     if (m < g.M) {
       const int b = m / g.HoWo, rem = m - b * g.HoWo;
       const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
@@ -107,6 +118,34 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
       iy0[i] = -(1 << 28);
       ix0[i] = 0;
       abase[i] = 0;
+    }
+  }
+  // GATHER_UNIFORM state.  The activation buffer starts (pt*W + pl)*Ci bytes before the
+  // input so that pixel offsets are non-negative; the weight buffer ends after row N-1,
+  // so rows past the last channel read as zeros.
+  [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc_a, rsrc_w;
+  [[maybe_unused]] unsigned poff[RA], pinv[RA], woff[RW];
+  [[maybe_unused]] int u_tap = 0, u_fx = 0, u_fy = 0, u_ci = 0, u_slice = 0;
+  if constexpr (UNI) {
+    const unsigned shift = (unsigned)((g.pt * g.W + g.pl) * g.Ci);
+    const unsigned batch = (unsigned)((g.M + g.HoWo - 1) / g.HoWo);
+    rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)(g.in - shift), 0, shift + batch * (unsigned)g.in_img, 0x00020000);
+    rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)g.w, 0, (unsigned)g.N * (unsigned)g.K, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < RA; i++) {
+      const int m = m0 + (tid >> 2) + RPP * i;
+      poff[i] = 0xffffffffu;
+      pinv[i] = 0;
+      if (m < g.M) {
+        const int b = m / g.HoWo, rem = m - b * g.HoWo;
+        const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
+        poff[i] = (unsigned)b * (unsigned)g.in_img + (unsigned)((oy * g.sy * g.W + ox * g.sx) * g.Ci) + 16u * ck;
+        for (int fy_ = 0, t = 0; fy_ < g.ky; fy_++)
+          for (int fx_ = 0; fx_ < g.kx; fx_++, t++) {
+            const int iy = oy * g.sy - g.pt + fy_, ix = ox * g.sx - g.pl + fx_;
+            if ((unsigned)iy >= (unsigned)g.H || (unsigned)ix >= (unsigned)g.W) pinv[i] |= 1u << t;
+          }
+      }
     }
   }
   // (fy, fx, ci) of byte k = 16*ck of the current K slice
@@ -123,27 +162,60 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
   int wpart[RW];
 #pragma unroll
   for (int i = 0; i < RW; i++) {
-    const int q = tid + 256 * i;
+    const int q = tid + NTH * i;
     const int p = q >> 2;
     wrow[i] = p;
     const int pp = p % WN, t = pp >> 4, r16 = pp & 15;
     wchan[i] = (p / WN) * WN + (r16 >> 2) * (4 * TN) + 4 * t + (r16 & 3);
     wact[i] = q < BN * 4;
     wpart[i] = 0;
+    if constexpr (UNI) {
+      const int n = n0 + wchan[i];
+      woff[i] = (wact[i] && n < g.N) ? (unsigned)n * (unsigned)g.K + 16u * ck : 0xffffffffu;
+    }
   }
 
-  // Two register sets: the loads of K slice kt+2 are in flight while slice kt is
-  // multiplied and slice kt+1 is staged, so a load has two slices of MFMA work to arrive.
+  // The loads of K slice kt+1 are in flight while slice kt is multiplied; they are staged
+  // into the other LDS buffer afterwards.  (A second register set for a two-slice distance
+  // costs 70 registers and with them a workgroup per CU, for no gain: the kernel is bound
+  // by LDS traffic, 48 KB per K slice and 128 x 128 tile, not by load latency.)
   struct Staged {
     v4i a[RA], w[RW];
     unsigned amask, wmask;  // bit i: chunk i holds real data (else it is staged as zero)
   };
-  Staged R0, R1;
+  Staged R0;
 
   // Issue the global loads of the next K slice.  Nothing here consumes a loaded value
   // (that would make the wave wait for it): out-of-image taps and out-of-range rows
   // load from a clamped, always valid address and are zeroed when staged into LDS.
   auto gload = [&](Staged &R) {
+    if constexpr (UNI) {
+      typedef unsigned v4u __attribute__((ext_vector_type(4)));
+      const int soff_a = (u_fy * g.W + u_fx) * g.Ci + u_ci;  // scalar: tap and channel offset of the slice
+      const int soff_w = u_slice * IGEMM_BK;
+#pragma unroll
+      for (int i = 0; i < RA; i++) {
+        // all ones if this tap is outside the image for this pixel
+        const unsigned oob = (unsigned)__builtin_amdgcn_sbfe((int)pinv[i], u_tap, 1);
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, poff[i] | oob, soff_a, 0);
+        R.a[i] = (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+      }
+#pragma unroll
+      for (int i = 0; i < RW; i++) {
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[i], soff_w, 0);
+        R.w[i] = (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+      }
+      R.amask = R.wmask = ~0u;
+      // advance to the next K slice (scalar)
+      u_slice++;
+      u_ci += IGEMM_BK;
+      if (u_ci >= g.Ci) {
+        u_ci = 0;
+        u_tap++;
+        if (++u_fx == g.kx) { u_fx = 0; ++u_fy; }
+      }
+      return;
+    }
     unsigned amask = 0, wmask = 0;
 #pragma unroll
     for (int i = 0; i < RA; i++) {
@@ -205,22 +277,26 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
 
   // Stage the loaded slice into LDS: activations as a ^ 0x80, invalid chunks as zero
   // (0x80 after the xor); weight bytes also feed the per-row sums.
-  auto sts = [&](const Staged &R, int buf) {
+  // live: the slice is one of the KT real ones (the prefetch runs up to two slices past
+  // the end; those are staged but never multiplied, and must not reach the weight sums).
+  auto sts = [&](const Staged &R, int buf, bool live) {
 #pragma unroll
     for (int i = 0; i < RA; i++) {
       v4i v = R.a[i];
-      if (!((R.amask >> i) & 1)) v = (v4i){0, 0, 0, 0};
-      *(v4i *)&As[buf][lds_off((tid >> 2) + 64 * i, ck)] = v ^ (int)0x80808080;
+      if (!UNI && !((R.amask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      *(v4i *)&As[buf][lds_off((tid >> 2) + RPP * i, ck)] = v ^ (int)0x80808080;
     }
 #pragma unroll
     for (int i = 0; i < RW; i++) {
       v4i v = R.w[i];
-      if (!((R.wmask >> i) & 1)) v = (v4i){0, 0, 0, 0};
+      if (!UNI && !((R.wmask >> i) & 1)) v = (v4i){0, 0, 0, 0};
       if (wact[i]) *(v4i *)&Ws[buf][lds_off(wrow[i], ck)] = v;
-      wpart[i] = __builtin_amdgcn_sdot4(v.x, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.y, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.z, 0x01010101, wpart[i], false);
-      wpart[i] = __builtin_amdgcn_sdot4(v.w, 0x01010101, wpart[i], false);
+      if (!UNI || live) {
+        wpart[i] = __builtin_amdgcn_sdot4(v.x, 0x01010101, wpart[i], false);
+        wpart[i] = __builtin_amdgcn_sdot4(v.y, 0x01010101, wpart[i], false);
+        wpart[i] = __builtin_amdgcn_sdot4(v.z, 0x01010101, wpart[i], false);
+        wpart[i] = __builtin_amdgcn_sdot4(v.w, 0x01010101, wpart[i], false);
+      }
     }
   };
 
@@ -248,23 +324,18 @@ __global__ __launch_bounds__(256, IGEMM_MINB) void igemm_kernel(ConvGeom g, EpiA
       for (int s = 0; s < TM; s++)
         acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[t], af[s], acc[t][s], 0, 0, 0);
   };
-  // Slices past the end load nothing (all-zero masks) and stage zeros: no branches needed.
+  // Slices past the end are loaded and staged but never multiplied: no branches needed.
+  // (The loop is kept rolled: unrolled by two it costs 60 more registers and a workgroup per CU.)
   gload(R0);
-  sts(R0, 0);
-  gload(R1);
+  sts(R0, 0, true);
   __syncthreads();
-  for (int kt = 0; kt < KT; kt += 2) {
-    gload(R0);        // slice kt + 2
-    compute(0);       // slice kt
-    sts(R1, 1);       // slice kt + 1
-    __syncthreads();
-    if (kt + 1 >= KT) break;
-    gload(R1);        // slice kt + 3
-    compute(1);       // slice kt + 1
-    sts(R0, 0);       // slice kt + 2
+#pragma unroll 1
+  for (int kt = 0; kt < KT; kt++) {
+    gload(R0);                            // slice kt + 1
+    compute(kt & 1);                      // slice kt
+    sts(R0, (kt + 1) & 1, kt + 1 < KT);
     __syncthreads();
   }
-
   // ---- per-row weight sums -> LDS (indexed by LDS row) ---------------------
 #pragma unroll
   for (int i = 0; i < RW; i++) {

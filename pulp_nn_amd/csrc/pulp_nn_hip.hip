@@ -79,7 +79,7 @@ void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   g.tiles_total = tiles_m * g.tiles_n;
   g.vec_store = (g.N % (4 * TN) == 0) && aligned(g.out, 4 * TN);
   g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
-  dim3 grid(g.tiles_total), block(256);
+  dim3 grid(g.tiles_total), block(64 * WM_ * WN_);
   switch (mode) {
     case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN, TM>), grid, block, 0, s, g, e); break;
     case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT, TM>), grid, block, 0, s, g, e); break;
@@ -100,7 +100,14 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
   const bool chunk16 = (g.Ci % 16 == 0) && aligned(g.in, 16) && aligned(g.w, 16);
-  if (chunk16) launch_igemm_tile<GATHER_CHUNK16>(mode, g, e, s);
+  // scalar tap walk + range-checked buffer loads: whole K slices inside one tap, one bit
+  // per tap in a 32-bit mask, 32-bit byte offsets
+  const long long batch = (g.M + g.HoWo - 1) / g.HoWo;
+  const bool uniform = chunk16 && (g.Ci % 64 == 0) && g.kx * g.ky <= 32 &&
+                       batch * g.in_img + (long long)(g.pt * g.W + g.pl) * g.Ci < 0x7fffffffLL &&
+                       (long long)g.N * g.K < 0x7fffffffLL;
+  if (uniform) launch_igemm_tile<GATHER_UNIFORM>(mode, g, e, s);
+  else if (chunk16) launch_igemm_tile<GATHER_CHUNK16>(mode, g, e, s);
   else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
 }
 
