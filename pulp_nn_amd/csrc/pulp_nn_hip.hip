@@ -21,6 +21,7 @@
 #include "pool.h"
 #include "pw_stream.h"
 #include "requant.h"
+#include "smallk.h"
 
 namespace {
 
@@ -109,6 +110,20 @@ void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   if (uniform) launch_igemm_tile<GATHER_UNIFORM>(mode, g, e, s);
   else if (chunk16) launch_igemm_tile<GATHER_CHUNK16>(mode, g, e, s);
   else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
+}
+
+// Direct (vector ALU) convolution for filters of at most 32 bytes and at most 32 channels.
+template <int NCH>
+void launch_smallk(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  g.vec_store = (g.N == NCH) && aligned(g.out, 16);
+  g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
+  dim3 grid((unsigned)((g.M + 255) / 256)), block(256);
+  switch (mode) {
+    case EPI_BN: hipLaunchKernelGGL((smallk_conv_kernel<NCH, EPI_BN>), grid, block, 0, s, g, e); break;
+    case EPI_MULT: hipLaunchKernelGGL((smallk_conv_kernel<NCH, EPI_MULT>), grid, block, 0, s, g, e); break;
+    default: hipLaunchKernelGGL((smallk_conv_kernel<NCH, EPI_RAW>), grid, block, 0, s, g, e); break;
+  }
 }
 
 int num_cus()
@@ -261,7 +276,12 @@ void conv_common(const char *fn, bool pointwise, const uint8_t *in, const int8_t
   g.sx = sx;
   g.sy = sy;
   g.in_img = (long long)dim_in_x * dim_in_y * ch_in;
-  launch_igemm(mode, g, e, g_stream);
+  if (g.K <= 4 * SMALLK_KD && g.N <= 32) {
+    if (g.N <= 16) launch_smallk<16>(mode, g, e, g_stream);
+    else launch_smallk<32>(mode, g, e, g_stream);
+  } else {
+    launch_igemm(mode, g, e, g_stream);
+  }
   check_launch(fn);
 }
 
