@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA, op/s
 PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
+HBM_TRAFFIC_CFG1 = int((12727.8 * 2.0 + 50185.3) * 1024)   # measured: FETCH_SIZE 12727.8 KiB x 2.0 + WRITE_SIZE 50185.3 KiB
 
 
 def main():
@@ -37,8 +38,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); the path shards by batch "
-                 "with no exchange, see DESIGN.md")
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1): every layer is independent per image, so "
+                 "more GPUs would each take a slice of the batch with no exchange; no multi-GPU figure is produced")
 
     import numpy as np
     import torch
@@ -103,7 +104,7 @@ def main():
 
     gops = c1["ops"] / (wall_ms * 1e-3) / 1e9
     rec = {
-        "metric": "int8 GOPS (2xMAC) on the pointwise conv layer at batch 256; bit-exact",
+        "metric": "int8 GOPS and % int8 MFMA peak per conv layer at batch 256; bit-exact",
         "value": round(gops, 1),
         "unit": "GOPS",
         "n_gpus": 1,
@@ -124,13 +125,16 @@ def main():
         "mfma_frac": round(c1["ops"] / (dev_ms * 1e-3) / PEAK_INT8_OPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "pw_stream_kernel<4, 2, 1, true, 2> (weights-stationary pointwise, scalar-multiplier epilogue)",
+            "kernel": "pw_stream_kernel<4, 2, 4, 1, true, 2, 8> (weights-stationary pointwise, scalar-multiplier "
+                      "epilogue)",
             "achieved": round(c1["bytes"] / (dev_ms * 1e-3) / 1e9, 1),
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
             "frac": round(c1["bytes"] / (dev_ms * 1e-3) / PEAK_HBM, 4),
             "algorithmic_bytes_per_launch": c1["bytes"],
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x 2.0, the factor a plain copy of known
+            # size shows for that counter) and WRITE_SIZE (x 1.0): profiles/bench_all_layers_hbm_traffic.txt
+            "traffic": HBM_TRAFFIC_CFG1,
         },
     }
 
