@@ -46,6 +46,11 @@ struct DwGeom {
   int in_align4;  // input pointer and W are multiples of 4: aligned dword loads are safe
   int out_vec4;   // output pointer and CH are multiples of 4: dword stores are safe
   int nt;         // write the output with non-temporal stores
+  // Packing of layers with fewer than 64 channels (dw3x3_lin_kernel only): CH and B describe the
+  // input re-read as images of 64 planes (CHW images lie back to back, so that is the same memory);
+  // CHR is the real channel count, planes the real number of planes B_real * CHR.
+  int CHR;
+  long long planes;
 };
 
 #define DW_CG 64  // channels per workgroup (one per lane)
@@ -363,15 +368,14 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   // ---- stage -----------------------------------------------------------------
   const int r_lo = max(0, -iy_start), r_hi = min(g.NR, g.H - iy_start);  // rows of the band inside the image
   const int run_len = max(r_hi - r_lo, 0) * g.W;                        // bytes per channel
-  const uint8_t *img = g.in + (long long)b * g.CH * g.H * g.W;
   const bool two = run_len + 12 > 64 * 16;  // a run may need more than 64 chunks
   {
     v4i ld[16][2];
     int mis[16];
 #pragma unroll
     for (int cc = 0; cc < 16; cc++) {
-      const int ch = min(c0 + wave + 4 * cc, g.CH - 1);
-      const uint8_t *g0 = img + ((long long)ch * g.H + min(max(iy_start + r_lo, 0), g.H - 1)) * g.W;
+      const long long pl_ = min((long long)b * g.CH + min(c0 + wave + 4 * cc, g.CH - 1), g.planes - 1);
+      const uint8_t *g0 = g.in + (pl_ * g.H + min(max(iy_start + r_lo, 0), g.H - 1)) * g.W;
       mis[cc] = (int)((uintptr_t)g0 & 15);
       const int last = max(((run_len + mis[cc] + 15) >> 4) - 1, 0);
       // lanes past the end of the run re-read its last chunk (masked off below)
@@ -382,7 +386,7 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
     for (int cc = 0; cc < 16; cc++) {
       const int c = wave + 4 * cc;
       const int dst = c * g.CSD + r_lo * LWD;
-      const unsigned keep = (c0 + c < g.CH) ? 0xFFFFFFFFu : 0u;
+      const unsigned keep = (c0 + c < g.CH && (long long)b * g.CH + c0 + c < g.planes) ? 0xFFFFFFFFu : 0u;
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         if (t == 1 && !two) break;
@@ -402,8 +406,8 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   }
 
   // ---- per-lane channel constants ------------------------------------------------
-  const int ch = c0 + lane;
-  const bool ch_ok = ch < g.CH;
+  const bool ch_ok = c0 + lane < g.CH && (long long)b * g.CH + c0 + lane < g.planes;
+  const int ch = (c0 + lane) % g.CHR;  // real channel: index of the weights and constants
   unsigned wA[3], wB[3];
   int corr = 0;
   bn_t kk = 0, ll = 0;
@@ -435,7 +439,7 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   DwColumn col;
   col.LWD = LWD;
   col.rows = rows;
-  col.row_bytes = (long long)g.Wo * g.CH;
+  col.row_bytes = (long long)g.Wo * g.CHR;
   col.corr = corr;
   col.k = kk;
   col.lambda = ll;
@@ -455,10 +459,13 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   for (int xg = wave; xg < xgroups; xg += 4) {
     col.dc0 = xg * S - 1;  // dword column of the first dword of the window
     col.p = lbase + xg * S;
-    col.o = g.out + (((long long)b * g.Ho + oy0) * g.Wo + 4 * xg + (lane & 3)) * g.CH + c0 + cq;
+    // this lane stores 4 consecutive channels of one pixel: plane pq .. pq+3 -> image pq / CHR, channel pq % CHR
+    const long long pq = (long long)b * g.CH + c0 + cq;
+    col.o = g.out + (((pq / g.CHR) * g.Ho + oy0) * g.Wo + 4 * xg + (lane & 3)) * g.CHR + (int)(pq % g.CHR);
     // 0: store a dword, 1: store the valid bytes one by one, 2: nothing to store
-    col.store = (4 * xg + (lane & 3) >= g.Wo) ? 2 : ((g.out_vec4 && c0 + cq + 3 < g.CH) ? 0 : 1);
-    col.nbytes = min(4, g.CH - c0 - cq);
+    const long long left = min((long long)(g.CH - c0 - cq), g.planes - pq);  // planes this lane may write
+    col.store = (4 * xg + (lane & 3) >= g.Wo || left <= 0) ? 2 : ((g.out_vec4 && left >= 4) ? 0 : 1);
+    col.nbytes = (int)min(4ll, max(left, 0ll));
     const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
     if (FULL && fastq && g.nt) {
       // one more copy of the common case for the streaming store policy

@@ -371,7 +371,14 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.bands = (Ho + g.RB - 1) / g.RB;
   g.NR = (g.RB - 1) * sy + ky;
   g.CSD = (g.NR * g.LWD) | 1;
-  g.cgroups = (CH + DW_CG - 1) / DW_CG;
+  g.CHR = CH;
+  g.planes = (long long)g.B * CH;
+  if (lin && CH < DW_CG && DW_CG % CH == 0 && CH % 4 == 0) {
+    // fewer than 64 channels: 64 / CH images share a workgroup (one plane per lane)
+    g.CH = DW_CG;
+    g.B = (int)((g.planes + DW_CG - 1) / DW_CG);
+  }
+  g.cgroups = (g.CH + DW_CG - 1) / DW_CG;
   const long long total = (long long)g.B * g.bands * g.cgroups;
   if (total > 0x7fffffffLL) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
   g.total = (int)total;
@@ -381,7 +388,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.inc_c = carry / g.NR;
   g.in_align4 = aligned(in, 4) && (W % 4 == 0);
   g.out_vec4 = aligned(out, 4) && (CH % 4 == 0);
-  g.nt = (long long)g.B * Ho * Wo * CH >= PULPNN_NT_BYTES;
+  g.nt = g.planes * Ho * Wo >= PULPNN_NT_BYTES;
   const size_t lds = (size_t)DW_CG * g.CSD * 4;
   dim3 grid(g.total), block(256);
 #define DW_LAUNCH(KERNEL)                                                                   \
@@ -392,7 +399,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   }
 #define DW3(S, PL, M) dw3x3_kernel<S, PL, M>
   if (lin) {
-    const bool full = (Wo % 4 == 0) && (CH % DW_CG == 0) && g.out_vec4;
+    const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
 #define DW3L_MODE(S, PL, FULL)                                                                                        \
   switch (mode) {                                                                                                     \

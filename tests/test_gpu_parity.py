@@ -132,6 +132,10 @@ DW_GEOMS = [
     (1, 5, 9, 9, 3, 3, (0, 0, 0, 0), (1, 1)),        # no padding: pl = 0 fast path
     (1, 5, 11, 11, 3, 3, (0, 0, 0, 0), (2, 2)),
     (1, 4, 10, 230, 3, 3, (1, 1, 1, 1), (1, 1)),     # wide image: few rows per band
+    (8, 16, 16, 16, 3, 3, (1, 1, 1, 1), (1, 1)),     # 16 channels: four images share a workgroup
+    (3, 16, 20, 16, 3, 3, (1, 1, 1, 1), (2, 2)),     # ... with a partly filled last group of images
+    (5, 32, 12, 24, 3, 3, (1, 1, 1, 1), (2, 2)),     # 32 channels: two images per workgroup, odd batch
+    (9, 8, 18, 20, 3, 3, (0, 0, 0, 0), (1, 1)),      # 8 channels: eight images per workgroup, no padding
 ]
 
 
@@ -156,7 +160,8 @@ def test_depthwise_generic(geom, flags, bn_bits):
 
 @pytest.mark.parametrize("bn_bits", [32, 64])
 @pytest.mark.parametrize("flags", [(1, 1), (1, 0), (0, 0)])
-@pytest.mark.parametrize("shape", [(2, 128, 56, 56), (2, 5, 7, 6), (1, 3, 1, 2), (3, 66, 12, 20)])
+@pytest.mark.parametrize("shape", [(2, 128, 56, 56), (2, 5, 7, 6), (1, 3, 1, 2), (3, 66, 12, 20), (6, 16, 12, 16),
+                                   (3, 32, 9, 20)])
 def test_depthwise_3x3_s1(shape, flags, bn_bits):
     B, CH, H, W = shape
     relu, bn = flags
