@@ -77,7 +77,8 @@ __device__ __forceinline__ int lds_off(int row, int chunk)
 }
 
 template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, WAVES_M * WAVES_N > 4 ? 1 : (GATHER == GATHER_BYTES ? 2 : IGEMM_MINB))
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N,
+                            (WAVES_M * WAVES_N > 8 || TM > 4) ? 1 : (WAVES_M * WAVES_N > 4 || GATHER == GATHER_BYTES ? 2 : IGEMM_MINB))
 void igemm_kernel(ConvGeom g, EpiArgs e)
 {
   constexpr int WM = 16 * TM, WN = 16 * TN;

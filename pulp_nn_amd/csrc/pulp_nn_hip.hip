@@ -69,6 +69,18 @@ bool epi_args(int mode, const bn_t *k, const bn_t *lambda, uint16_t out_mult, in
   return e->shift >= 0 && e->shift < lim;
 }
 
+int num_cus()
+{
+  static int n = 0;
+  if (!n) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+
 // ---- implicit GEMM dispatch -------------------------------------------------
 
 template <int TN, int WM_, int WN_, int GATHER, int TM = 4>
@@ -94,6 +106,11 @@ void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 template <int GATHER>
 void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
+  // 256 px x 256 ch with 16 waves when there are at least two such tiles per CU: half the
+  // L2 -> LDS bytes per multiply of the 128 x 128 tile
+  const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
+  if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
+  else
   if (g.N > 64) launch_igemm_mode<4, 2, 2, GATHER>(mode, g, e, s);       // 128 px x 128 ch
   else if (g.N > 32) launch_igemm_mode<4, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 64 ch
   else if (g.N > 16) launch_igemm_mode<2, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 32 ch
@@ -128,17 +145,6 @@ void launch_smallk(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   }
 }
 
-int num_cus()
-{
-  static int n = 0;
-  if (!n) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
-    if (n <= 0) n = 256;
-  }
-  return n;
-}
 
 #ifndef PW_NW
 #define PW_NW 8  // waves per workgroup of the streaming kernel
