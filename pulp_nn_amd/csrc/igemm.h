@@ -93,6 +93,9 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   __shared__ __attribute__((aligned(16))) uint8_t As[2][BM * IGEMM_BK];
   __shared__ __attribute__((aligned(16))) int8_t Ws[2][BN * IGEMM_BK];
   __shared__ int wsum[BN];
+  // per-channel constants of the tile, fetched while the first K slice is on its way
+  __shared__ int cbias[BN];
+  __shared__ bn_t ck_[MODE == EPI_BN ? BN : 1], cl_[MODE == EPI_BN ? BN : 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -327,6 +330,23 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   };
   // Slices past the end are loaded and staged but never multiplied: no branches needed.
   // (The loop is kept rolled: unrolled by two it costs 60 more registers and a workgroup per CU.)
+  for (int c = tid; c < BN; c += NTH) {
+    const int n = n0 + c;
+    int b = 0;
+    bn_t kv = 0, lv = 0;
+    if (n < g.N) {
+      if (g.bias) b = (MODE == EPI_OUT32) ? ((const int *)g.bias)[n] : (int)g.bias[n];
+      if (MODE == EPI_BN) {
+        kv = e.k[n];
+        lv = e.lambda[n];
+      }
+    }
+    cbias[c] = b;
+    if (MODE == EPI_BN) {
+      ck_[c] = kv;
+      cl_[c] = lv;
+    }
+  }
   gload(R0);
   sts(R0, 0, true);
   __syncthreads();
@@ -362,19 +382,11 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
     bool ks = true;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      const int n = n0 + cb + 4 * t + r;
-      int b = 0;
-      kk[r] = 0;
-      ll[r] = 0;
-      if (n < g.N) {
-        if (g.bias) b = (MODE == EPI_OUT32) ? ((const int *)g.bias)[n] : (int)g.bias[n];
-        if (MODE == EPI_BN) {
-          kk[r] = e.k[n];
-          ll[r] = e.lambda[n];
-        }
-      }
+      const int c = cb + 4 * t + r;  // channel inside the tile (constants of channels past N are zero)
+      kk[r] = (MODE == EPI_BN) ? ck_[c] : (bn_t)0;
+      ll[r] = (MODE == EPI_BN) ? cl_[c] : (bn_t)0;
       ks = ks && bn_k_small(kk[r]);
-      corr[r] = b + 128 * wsum[wave_n * WN + 16 * t + 4 * lgrp + r];
+      corr[r] = cbias[c] + 128 * wsum[wave_n * WN + 16 * t + 4 * lgrp + r];
     }
     const bool k_small = __all(ks);  // wave-uniform precondition of the fast batch-norm form
 #pragma unroll
