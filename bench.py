@@ -125,7 +125,7 @@ def main():
         "mfma_frac": round(c1["ops"] / (dev_ms * 1e-3) / PEAK_INT8_OPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "pw_stream_kernel<4, 2, 4, 1, true, 2, 8> (weights-stationary pointwise, scalar-multiplier "
+            "kernel": "pw_stream_kernel<4, 2, 4, 1, true, 1, 16> (weights-stationary pointwise, scalar-multiplier "
                       "epilogue)",
             "achieved": round(c1["bytes"] / (dev_ms * 1e-3) / 1e9, 1),
             "peak": PEAK_HBM / 1e9,

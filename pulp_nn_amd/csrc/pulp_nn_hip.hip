@@ -146,16 +146,6 @@ void launch_smallk(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 }
 
 
-#ifndef PW_NW
-#define PW_NW 8  // waves per workgroup of the streaming kernel
-#endif
-#ifndef PW_TM
-#define PW_TM 2  // 16-pixel units per step
-#endif
-#ifndef PW_PER_CU
-#define PW_PER_CU 1
-#endif
-
 // Launches one instantiation; raises its dynamic-LDS limit above the default 64 KB as needed.
 template <auto KERN>
 void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t lds, hipStream_t s)
@@ -168,10 +158,14 @@ void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t 
   hipLaunchKernelGGL(KERN, grid, block, lds, s, g, e);
 }
 
-template <int TN, int NP, int KS>
+// Two shapes of the streaming kernel: 16 waves taking 16 pixels per step for launches
+// with at least three steps for every wave of every CU (more waves in flight hide the
+// arithmetic of a step behind the memory traffic of the others), 8 waves taking 32 pixels
+// per step otherwise (half the LDS reads per pixel, and the 128-register budget of the
+// 16-wave shape is too small for K = 256).
+template <int TN, int NP, int KS, int TM, int NW>
 void launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
 {
-  constexpr int TM = PW_TM, NW = PW_NW;
   dim3 block(64 * NW);
   switch (mode) {
     case EPI_BN: launch_pw<pw_stream_kernel<TN, KS, NP, EPI_BN, false, TM, NW>>(g, e, grid, block, lds, s); break;
@@ -184,11 +178,18 @@ void launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 gri
 }
 
 template <int TN, int NP>
-void launch_pw_stream_ks(int mode, int ks, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
+void launch_pw_stream_ks(int mode, int ks, bool wide, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds,
+                         hipStream_t s)
 {
-  if (ks == 1) launch_pw_stream_mode<TN, NP, 1>(mode, g, e, grid, lds, s);
-  else if (ks == 2) launch_pw_stream_mode<TN, NP, 2>(mode, g, e, grid, lds, s);
-  else launch_pw_stream_mode<TN, NP, 4>(mode, g, e, grid, lds, s);
+  if (ks == 1) {
+    if (wide) launch_pw_stream_mode<TN, NP, 1, 1, 16>(mode, g, e, grid, lds, s);
+    else launch_pw_stream_mode<TN, NP, 1, 2, 8>(mode, g, e, grid, lds, s);
+  } else if (ks == 2) {
+    if (wide) launch_pw_stream_mode<TN, NP, 2, 1, 16>(mode, g, e, grid, lds, s);
+    else launch_pw_stream_mode<TN, NP, 2, 2, 8>(mode, g, e, grid, lds, s);
+  } else {
+    launch_pw_stream_mode<TN, NP, 4, 2, 8>(mode, g, e, grid, lds, s);
+  }
 }
 
 // Weights-stationary streaming path: a GEMM whose rows are contiguous K-byte pixels,
@@ -213,22 +214,24 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   g.M = (int)M;
   g.N = N;
   g.K = K;
-  const int lds = pw_lds_bytes(tn, ks, np, mode == EPI_BN, PW_NW, PW_TM);
-  if (lds > (160 * 1024 - 512) / PW_PER_CU) return false;  // 512: static LDS of the kernel
   g.units = (int)((M + 15) / 16);
   g.nt = M * N >= PULPNN_NT_BYTES;
+  const bool wide = ks <= 2 && g.units >= 3 * 16 * num_cus();
+  const int nw = wide ? 16 : 8, tm = wide ? 1 : 2;
+  const int lds = pw_lds_bytes(tn, ks, np, mode == EPI_BN, nw, tm);
+  if (lds > 160 * 1024 - 512) return false;  // 512: static LDS of the kernel
   // Persistent grid: one workgroup per CU (the weights are staged once per CU), fewer
   // when there are not two 16-pixel units for every wave.
-  int blocks = PW_PER_CU * num_cus();
-  const int need = (g.units + 2 * PW_NW - 1) / (2 * PW_NW);
+  int blocks = num_cus();
+  const int need = (g.units + 2 * nw - 1) / (2 * nw);
   if (blocks > need) blocks = need;
   dim3 grid(blocks);
-  if (tn == 1) launch_pw_stream_ks<1, 1>(mode, ks, g, e, grid, lds, s);
-  else if (tn == 2) launch_pw_stream_ks<2, 1>(mode, ks, g, e, grid, lds, s);
-  else if (np == 1) launch_pw_stream_ks<4, 1>(mode, ks, g, e, grid, lds, s);
-  else if (np == 2) launch_pw_stream_ks<4, 2>(mode, ks, g, e, grid, lds, s);
-  else if (np == 3) launch_pw_stream_ks<4, 3>(mode, ks, g, e, grid, lds, s);
-  else launch_pw_stream_ks<4, 4>(mode, ks, g, e, grid, lds, s);
+  if (tn == 1) launch_pw_stream_ks<1, 1>(mode, ks, wide, g, e, grid, lds, s);
+  else if (tn == 2) launch_pw_stream_ks<2, 1>(mode, ks, wide, g, e, grid, lds, s);
+  else if (np == 1) launch_pw_stream_ks<4, 1>(mode, ks, wide, g, e, grid, lds, s);
+  else if (np == 2) launch_pw_stream_ks<4, 2>(mode, ks, wide, g, e, grid, lds, s);
+  else if (np == 3) launch_pw_stream_ks<4, 3>(mode, ks, wide, g, e, grid, lds, s);
+  else launch_pw_stream_ks<4, 4>(mode, ks, wide, g, e, grid, lds, s);
   return true;
 }
 

@@ -75,10 +75,23 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
   unsigned char *ob = pw_lds + pw_lds_fixed(TN, KS, NP, MODE == EPI_BN) + wave * (PX * OROW);
 
   // ---- this wave's share of the pixels ---------------------------------------------------
-  // This wave's pixels: an equal share of the 16-pixel units, contiguous in memory.
-  const int nwaves = gridDim.x * NW, gw = blockIdx.x * NW + wave;
-  const int px_end = min((int)((long long)g.units * (gw + 1) / nwaves) * 16, g.M);
-  int px = (int)((long long)g.units * gw / nwaves) * 16;
+  // A quarter of the waves stages the weights; the others request their first pixels at
+  // once, have them by the time the weights are in place and so start streaming about one
+  // step earlier.  The 16-pixel units of the launch are dealt evenly to the
+  // workgroups and, inside a workgroup, one step's worth (TM units) fewer to each staging
+  // wave than the average and the rest evenly to the others, all in contiguous runs, so
+  // that all waves finish together.
+  constexpr int NWS = NW >= 4 ? NW / 4 : 1;  // staging waves
+  const bool stager = wave < NWS;
+  const int ub0 = (int)((long long)g.units * blockIdx.x / gridDim.x);
+  const int nb = (int)((long long)g.units * (blockIdx.x + 1) / gridDim.x) - ub0;  // units of this workgroup
+  // (no handicap when a wave has fewer than three steps anyway: the set-up then dominates)
+  const int us = nb / NW >= 3 * TM ? nb / NW - TM : nb / NW;                      // units of a staging wave
+  const int rest = nb - NWS * us;                                                 // units of the other waves
+  const int u_beg = stager ? wave * us : NWS * us + (int)((long long)rest * (wave - NWS) / (NW - NWS));
+  const int u_end = stager ? (wave + 1) * us : NWS * us + (int)((long long)rest * (wave - NWS + 1) / (NW - NWS));
+  const int px_end = min((ub0 + u_end) * 16, g.M);
+  int px = (ub0 + u_beg) * 16;
   // Unconditional loads from clamped addresses (no per-lane branches, so that all
   // loads of a step are issued back to back and nothing waits on them here):
   // pixels past the end of the run re-read its last pixel and K chunks past the end
@@ -97,54 +110,61 @@ __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwG
   };
   v4i b0[TM][KS], b1[TM][KS], b2[TM][KS];
 
-  // ---- weights and per-channel constants -> LDS -----------------------------------
-  // All global loads of the set-up are issued before the first of them is consumed.
-  constexpr int CHUNKS = N * KS * 4;             // 16-byte chunks of the padded weight matrix
-  constexpr int CH = (CHUNKS + BS - 1) / BS;     // per thread
-  constexpr int NC = (N + BS - 1) / BS;          // channels per thread
-  v4i wv[CH];
-#pragma unroll
-  for (int u = 0; u < CH; u++) {
-    // LDS row R = ((p*KS + ks)*TN + t)*16 + i holds channel p*CG + (i/4)*4*TN + 4*t + i%4
-    const int q = tid + BS * u, R = q >> 2, c = q & 3;
-    const int i = R & 15, t = (R >> 4) % TN, ks = (R / CG) % KS, p = R / (CG * KS);
-    const int n = p * CG + (i >> 2) * (4 * TN) + 4 * t + (i & 3);
-    const int k = ks * 64 + 16 * c;
-    const bool ok = q < CHUNKS && k < g.K;
-    wv[u] = *(const v4i *)(g.w + (ok ? (long long)n * g.K + k : 0));
+  if (!stager) {
+    load_a(b0, px);
+    load_a(b1, px + PX);
   }
-  int bv[NC];
-  bn_t kv[NC], lv[NC];
-#pragma unroll
-  for (int u = 0; u < NC; u++) {
-    const int n = min(tid + BS * u, N - 1);
-    bv[u] = g.bias ? (int)g.bias[n] : 0;
-    if constexpr (MODE == EPI_BN) {
-      kv[u] = e.k[n];
-      lv[u] = e.lambda[n];
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < CH; u++) {
-    const int q = tid + BS * u, R = q >> 2, c = q & 3;
-    const int k = ((R / CG) % KS) * 64 + 16 * c;
-    if (q < CHUNKS) *(v4i *)&Wl[lds_off(R, c)] = (k < g.K) ? wv[u] : (v4i){0, 0, 0, 0};
-  }
-  // The first two steps' pixels are requested only now: the CU's memory pipeline serves
-  // requests in order, and the (few, mostly L2-resident) set-up loads are not to queue
-  // behind 64 KB of pixels from HBM.
-  load_a(b0, px);
-  load_a(b1, px + PX);
+  // ---- weights and per-channel constants -> LDS (staging waves) -------------------------
   bool small = true;
+  if (stager) {
+    // All global loads of the set-up are issued before the first of them is consumed.
+    constexpr int SB = 64 * NWS;                   // staging threads
+    constexpr int CHUNKS = N * KS * 4;             // 16-byte chunks of the padded weight matrix
+    constexpr int CH = (CHUNKS + SB - 1) / SB;     // per thread
+    constexpr int NC = (N + SB - 1) / SB;          // channels per thread
+    v4i wv[CH];
 #pragma unroll
-  for (int u = 0; u < NC; u++) {
-    const int n = tid + BS * u;
-    if (n < N) {
-      corr_l[n] = bv[u];
+    for (int u = 0; u < CH; u++) {
+      // LDS row R = ((p*KS + ks)*TN + t)*16 + i holds channel p*CG + (i/4)*4*TN + 4*t + i%4
+      const int q = tid + SB * u, R = q >> 2, c = q & 3;
+      const int i = R & 15, t = (R >> 4) % TN, ks = (R / CG) % KS, p = R / (CG * KS);
+      const int n = p * CG + (i >> 2) * (4 * TN) + 4 * t + (i & 3);
+      const int k = ks * 64 + 16 * c;
+      const bool ok = q < CHUNKS && k < g.K;
+      wv[u] = *(const v4i *)(g.w + (ok ? (long long)n * g.K + k : 0));
+    }
+    int bv[NC];
+    bn_t kv[NC], lv[NC];
+#pragma unroll
+    for (int u = 0; u < NC; u++) {
+      const int n = min(tid + SB * u, N - 1);
+      bv[u] = g.bias ? (int)g.bias[n] : 0;
       if constexpr (MODE == EPI_BN) {
-        kl[n] = kv[u];
-        ll_[n] = lv[u];
-        small = small && bn_k_small(kv[u]);
+        kv[u] = e.k[n];
+        lv[u] = e.lambda[n];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < CH; u++) {
+      const int q = tid + SB * u, R = q >> 2, c = q & 3;
+      const int k = ((R / CG) % KS) * 64 + 16 * c;
+      if (q < CHUNKS) *(v4i *)&Wl[lds_off(R, c)] = (k < g.K) ? wv[u] : (v4i){0, 0, 0, 0};
+    }
+    // The staging waves request their first two steps only now: the CU's memory pipeline
+    // serves requests in order, and their (few, mostly L2-resident) set-up loads were not
+    // to queue behind their own pixels from HBM.
+    load_a(b0, px);
+    load_a(b1, px + PX);
+#pragma unroll
+    for (int u = 0; u < NC; u++) {
+      const int n = tid + SB * u;
+      if (n < N) {
+        corr_l[n] = bv[u];
+        if constexpr (MODE == EPI_BN) {
+          kl[n] = kv[u];
+          ll_[n] = lv[u];
+          small = small && bn_k_small(kv[u]);
+        }
       }
     }
   }

@@ -85,6 +85,8 @@ PW_GEOMS = [
     (3, 30, 30, 32, 16),     # N = 16
     (2, 40, 40, 64, 64),     # one channel group
     (2, 33, 35, 64, 128),    # two channel groups, pixel count not a multiple of 64
+    (16, 112, 112, 32, 64),  # 200704 pixels: the 16-wave shape of the streaming kernel, one channel group
+    (16, 112, 113, 16, 32),  # ... 32 channels, pixel count not a multiple of 16 per wave
     (16, 65, 64, 64, 300),   # 66560 pixels x 300 channels: the 256 x 256 tiles of the tiled kernel, channel tail
     (2, 33, 33, 256, 200),   # K = 256, channel tail inside the last group
     (2, 40, 30, 48, 100),    # K and N not multiples of 64
