@@ -346,9 +346,13 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
 //
 // FULL: Wo % 4 == 0, CH % 64 == 0 and the output is 4-byte aligned, so every lane
 // stores one dword per output row without any bounds check.
+#ifndef DW_WAVES
+#define DW_WAVES 8  // waves per workgroup of dw3x3_lin_kernel
+#endif
 template <int S, int PL, int MODE, bool FULL>
-__global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
+__global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
 {
+  constexpr int NWV = DW_WAVES, CPW = DW_CG / NWV;  // waves, channels staged per wave
   extern __shared__ unsigned dw_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -370,11 +374,11 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   const int run_len = max(r_hi - r_lo, 0) * g.W;                        // bytes per channel
   const bool two = run_len + 12 > 64 * 16;  // a run may need more than 64 chunks
   {
-    v4i ld[16][2];
-    int mis[16];
+    v4i ld[CPW][2];
+    int mis[CPW];
 #pragma unroll
-    for (int cc = 0; cc < 16; cc++) {
-      const long long pl_ = min((long long)b * g.CH + min(c0 + wave + 4 * cc, g.CH - 1), g.planes - 1);
+    for (int cc = 0; cc < CPW; cc++) {
+      const long long pl_ = min((long long)b * g.CH + min(c0 + wave + NWV * cc, g.CH - 1), g.planes - 1);
       const uint8_t *g0 = g.in + (pl_ * g.H + min(max(iy_start + r_lo, 0), g.H - 1)) * g.W;
       mis[cc] = (int)((uintptr_t)g0 & 15);
       const int last = max(((run_len + mis[cc] + 15) >> 4) - 1, 0);
@@ -383,8 +387,8 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
       if (two) ld[cc][1] = *(const v4i *)(g0 - mis[cc] + 16 * min(lane + 64, last));
     }
 #pragma unroll
-    for (int cc = 0; cc < 16; cc++) {
-      const int c = wave + 4 * cc;
+    for (int cc = 0; cc < CPW; cc++) {
+      const int c = wave + NWV * cc;
       const int dst = c * g.CSD + r_lo * LWD;
       const unsigned keep = (c0 + c < g.CH && (long long)b * g.CH + c0 + c < g.planes) ? 0xFFFFFFFFu : 0u;
 #pragma unroll
@@ -456,7 +460,7 @@ __global__ __launch_bounds__(256) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
   const bool fastq = (MODE == EPI_BN) ? k_small : (e.shift >= 16);
   constexpr int NS = ((4 - PL) + 3 * S + 2) / 4 + 1;
 
-  for (int xg = wave; xg < xgroups; xg += 4) {
+  for (int xg = wave; xg < xgroups; xg += NWV) {
     col.dc0 = xg * S - 1;  // dword column of the first dword of the window
     col.p = lbase + xg * S;
     // this lane stores 4 consecutive channels of one pixel: plane pq .. pq+3 -> image pq / CHR, channel pq % CHR

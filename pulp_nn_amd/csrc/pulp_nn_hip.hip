@@ -410,6 +410,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   if (lin) {
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
+    const dim3 block(64 * DW_WAVES);
 #define DW3L_MODE(S, PL, FULL)                                                                                        \
   switch (mode) {                                                                                                     \
     case EPI_BN: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_BN, FULL>), grid, block, ldsl, g_stream, g, e); break;     \
