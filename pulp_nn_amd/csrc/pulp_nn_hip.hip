@@ -112,6 +112,7 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
   else
   if (g.N > 64) launch_igemm_mode<4, 2, 2, GATHER>(mode, g, e, s);       // 128 px x 128 ch
+  else if (g.N > 32 && (g.M + 255) / 256 < 2 * num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);  // 128 px x 64 ch: more workgroups
   else if (g.N > 32) launch_igemm_mode<4, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 64 ch
   else if (g.N > 16) launch_igemm_mode<2, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 32 ch
   else launch_igemm_mode<1, 4, 1, GATHER>(mode, g, e, s);                // 256 px x 16 ch
