@@ -181,7 +181,8 @@ def test_depthwise_3x3_s1(shape, flags, bn_bits):
 
 
 @pytest.mark.parametrize("bn_bits", [32, 64])
-@pytest.mark.parametrize("dims", [(64, 1024, 4096), (256, 512, 1000), (3, 37, 11), (1, 512, 1000), (5, 100, 70)])
+@pytest.mark.parametrize("dims", [(64, 1024, 4096), (256, 512, 1000), (3, 37, 11), (1, 512, 1000), (5, 100, 70),
+                                  (70, 48, 30), (130, 256, 132), (300, 64, 64)])
 def test_linear(dims, bn_bits):
     B, K, N = dims
     r = rng_for(5000 + K)
@@ -193,7 +194,7 @@ def test_linear(dims, bn_bits):
         assert_same(linear(x, w, b, k, lam, 800, shift, relu, bn, bn_bits), want, "linear %d %d" % (relu, bn))
 
 
-@pytest.mark.parametrize("dims", [(256, 512, 1000), (3, 37, 11), (2, 1024, 64)])
+@pytest.mark.parametrize("dims", [(256, 512, 1000), (3, 37, 11), (2, 1024, 64), (100, 80, 20)])
 def test_linear_out_32(dims):
     B, K, N = dims
     r = rng_for(6000 + K)
