@@ -8,12 +8,13 @@
 // Every wave owns a contiguous run of pixels and streams it 16*TM pixels per step:
 // the activation bytes go from HBM straight into registers in the MFMA
 // column-operand layout (lane = pixel l%16, 16-byte K chunk l/16), each byte is
-// loaded by exactly one wave, and the loads run two steps ahead of the arithmetic;
-// the first two steps are requested before the weights are staged, so that HBM is
-// busy while the workgroup sets up.  A step multiplies its pixels against every
-// channel group, requantises, gathers the channel groups of a pixel in a per-wave
-// LDS tile and writes whole pixel rows, 1 KB contiguous per store instruction.
-// There is no barrier after the set-up and no im2col.
+// loaded by exactly one wave, and the loads run two steps ahead of the arithmetic.
+// A quarter of the waves stages the weights and constants; the others request the
+// pixels of their first two steps at once, so that HBM is busy while the workgroup
+// sets up.  A step multiplies its pixels against every channel group, requantises,
+// gathers the channel groups of a pixel in a per-wave LDS tile and writes whole
+// pixel rows, 1 KB contiguous per store instruction.  Two barriers end the set-up;
+// there is none in the streaming loop and no im2col.
 //
 // Everything the compiler has to count is fixed at compile time (loads and stores
 // per step, channel groups): loads and stores share one in-order counter on this
