@@ -133,13 +133,23 @@ void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
 }
 
-// Direct (vector ALU) convolution for filters of at most 32 bytes and at most 32 channels.
+// Direct (vector ALU) convolution for small filters and at most 32 channels.  rows: the filter
+// has at most 3 rows of at most 12 bytes and is gathered a row at a time (smallk_rows_kernel);
+// otherwise it is at most 32 bytes long and gathered byte by byte (smallk_conv_kernel).
 template <int NCH>
-void launch_smallk(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+void launch_smallk(int mode, bool rows, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
   g.vec_store = (g.N == NCH) && aligned(g.out, 16);
   g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
   dim3 grid((unsigned)((g.M + 255) / 256)), block(256);
+  if (rows) {
+    switch (mode) {
+      case EPI_BN: hipLaunchKernelGGL((smallk_rows_kernel<NCH, EPI_BN>), grid, block, 0, s, g, e); break;
+      case EPI_MULT: hipLaunchKernelGGL((smallk_rows_kernel<NCH, EPI_MULT>), grid, block, 0, s, g, e); break;
+      default: hipLaunchKernelGGL((smallk_rows_kernel<NCH, EPI_RAW>), grid, block, 0, s, g, e); break;
+    }
+    return;
+  }
   switch (mode) {
     case EPI_BN: hipLaunchKernelGGL((smallk_conv_kernel<NCH, EPI_BN>), grid, block, 0, s, g, e); break;
     case EPI_MULT: hipLaunchKernelGGL((smallk_conv_kernel<NCH, EPI_MULT>), grid, block, 0, s, g, e); break;
@@ -289,9 +299,15 @@ void conv_common(const char *fn, bool pointwise, const uint8_t *in, const int8_t
   g.sx = sx;
   g.sy = sy;
   g.in_img = (long long)dim_in_x * dim_in_y * ch_in;
-  if (g.K <= 4 * SMALLK_KD && g.N <= 32) {
-    if (g.N <= 16) launch_smallk<16>(mode, g, e, g_stream);
-    else launch_smallk<32>(mode, g, e, g_stream);
+  // a filter row is kx * ch_in contiguous input bytes: three aligned dwords cover it if it is at
+  // most 9 bytes long, or 12 with rows that start on a dword
+  const int row_bytes = (int)kx * ch_in;
+  const long long batch = (g.M + g.HoWo - 1) / g.HoWo;
+  const bool rows = ky <= 3 && (row_bytes <= 9 || (row_bytes <= 12 && ch_in % 4 == 0)) && aligned(g.in, 4) &&
+                    batch * g.in_img < 0x7ffffff0LL;
+  if ((rows || g.K <= 4 * SMALLK_KD) && g.N <= 32) {
+    if (g.N <= 16) launch_smallk<16>(mode, rows, g, e, g_stream);
+    else launch_smallk<32>(mode, rows, g, e, g_stream);
   } else {
     launch_igemm(mode, g, e, g_stream);
   }

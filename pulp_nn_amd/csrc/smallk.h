@@ -130,3 +130,144 @@ __global__ __launch_bounds__(256) void smallk_conv_kernel(ConvGeom g, EpiArgs e)
       if (n < g.N) o[n] = (uint8_t)(packed[n >> 2] >> (8 * (n & 3)));
   }
 }
+
+// The same for filters of at most 3 rows whose rows (kx * Ci bytes, contiguous in the HWC
+// input) are at most 9 bytes long, or at most 12 with Ci % 4 == 0: the 3x3 stem on RGB or
+// RGBA.  A filter row of a pixel is fetched as one range-checked 12-byte buffer load from the
+// aligned address below it (a row outside the image is an out-of-range load, which returns
+// zeros) and shifted into place, instead of byte by byte: 3 loads per pixel instead of 27.  Filter rows are padded
+// to 12 bytes in the weight table, so bytes past the end of a row meet zero weights; columns
+// outside the image are masked to zero.
+#define SMALLK_RD 3                  // dwords per filter row
+#define SMALLK_RP (3 * SMALLK_RD + 3)  // weight table pitch per channel (12 dwords: 16-byte reads)
+
+template <int NCH, int MODE>
+__global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
+{
+  __shared__ __attribute__((aligned(16))) int wl[NCH * SMALLK_RP];  // [channel][row][dword]
+  __shared__ int corr_l[NCH];
+  __shared__ bn_t k_l[NCH], lam_l[NCH];
+
+  const int tid = threadIdx.x;
+  const int L = g.kx * g.Ci;  // bytes per filter row
+  // ---- weights and constants -> LDS -------------------------------------------------
+  for (int q = tid; q < NCH * SMALLK_RP; q += 256) {
+    const int n = q / SMALLK_RP, d = q % SMALLK_RP, fy = d / SMALLK_RD, i = d % SMALLK_RD;
+    unsigned v = 0;
+    if (n < g.N && fy < g.ky) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int kk = 4 * i + j;
+        if (kk < L) v |= (unsigned)(uint8_t)g.w[(long long)n * g.K + fy * L + kk] << (8 * j);
+      }
+    }
+    wl[q] = (int)v;
+  }
+  __syncthreads();
+  if (tid < NCH) {
+    int sum = 0;
+#pragma unroll
+    for (int d = 0; d < 3 * SMALLK_RD; d++) sum = __builtin_amdgcn_sdot4(wl[tid * SMALLK_RP + d], 0x01010101, sum, false);
+    const bool real = tid < g.N;
+    corr_l[tid] = 128 * sum + ((real && g.bias) ? (int)g.bias[tid] : 0);
+    if (MODE == EPI_BN) {
+      k_l[tid] = real ? e.k[tid] : 0;
+      lam_l[tid] = real ? e.lambda[tid] : 0;
+    }
+  }
+  __syncthreads();
+
+  // ---- this lane's pixel: its (up to) three filter rows ------------------------------------
+  const int m = blockIdx.x * 256 + tid;
+  if (m >= g.M) return;
+  const int b = m / g.HoWo, rem = m - b * g.HoWo;
+  const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
+  const int iy0 = oy * g.sy - g.pt, ix0 = ox * g.sx - g.pl;
+  const unsigned batch = (unsigned)((g.M + g.HoWo - 1) / g.HoWo);
+  const int total = (int)(batch * (unsigned)g.in_img);  // bytes of input
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)g.in, 0, total, 0x00020000);
+  // bytes [lo, hi) of a filter row lie inside the image
+  const int lo = max(0, -ix0) * g.Ci, hi = max(min(g.kx, g.W - ix0), 0) * g.Ci;
+  const unsigned bits = ((1u << hi) - 1u) & ~((1u << lo) - 1u);  // hi <= 12
+  unsigned md[SMALLK_RD];
+#pragma unroll
+  for (int i = 0; i < SMALLK_RD; i++) md[i] = ((((bits >> (4 * i)) & 15u) * 0x00204081u) & 0x01010101u) * 0xFFu;
+  const int rowpos = (int)((unsigned)b * (unsigned)g.in_img) + ix0 * g.Ci;  // byte offset of the row's first byte, less iy * W * Ci
+  typedef unsigned v3u __attribute__((ext_vector_type(3)));
+  unsigned a[3][SMALLK_RD];
+#pragma unroll
+  for (int fy = 0; fy < 3; fy++) {
+    const int iy = iy0 + fy;
+    const bool ok = fy < g.ky && (unsigned)iy < (unsigned)g.H;
+    const int A = rowpos + iy * g.W * g.Ci;
+    const int sh = A & 3, base = A - sh;
+    // The 12 bytes from the aligned address below the row's first byte, as one range-checked
+    // load; a row outside the image is given an offset that is out of range, which loads zeros.
+    const v3u d = __builtin_amdgcn_raw_buffer_load_b96(rsrc, ok ? base : (int)0xfffffff0, 0, 0);
+    unsigned r0 = __builtin_amdgcn_alignbyte(d.y, d.x, sh);
+    unsigned r1 = __builtin_amdgcn_alignbyte(d.z, d.y, sh);
+    unsigned r2 = __builtin_amdgcn_alignbyte(0u, d.z, sh);
+    // The load must lie inside the input as a whole.  Where it would not (left padding in the
+    // first row of the first image, the last bytes of the last image), the few lanes concerned
+    // fetch the bytes of the row that lie inside the image one by one.
+    if (ok && (base < 0 || base + 12 > total)) {
+      unsigned t[SMALLK_RD] = {0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 4 * SMALLK_RD; j++)
+        if (j >= lo && j < hi) t[j >> 2] |= (unsigned)g.in[A + j] << (8 * (j & 3));
+      r0 = t[0];
+      r1 = t[1];
+      r2 = t[2];
+    }
+    a[fy][0] = (r0 & md[0]) ^ 0x80808080u;
+    a[fy][1] = (r1 & md[1]) ^ 0x80808080u;
+    a[fy][2] = (r2 & md[2]) ^ 0x80808080u;
+  }
+
+  // ---- NCH dot products, requantise, store ----------------------------------------------
+  unsigned packed[NCH / 4];
+#pragma unroll
+  for (int n4 = 0; n4 < NCH / 4; n4++) {
+    int acc[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int n = 4 * n4 + r;
+      acc[r] = corr_l[n];
+      const v4i w0 = *(const v4i *)&wl[n * SMALLK_RP], w1 = *(const v4i *)&wl[n * SMALLK_RP + 4];
+      const int w2 = wl[n * SMALLK_RP + 8];
+      acc[r] = __builtin_amdgcn_sdot4((int)a[0][0], w0.x, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[0][1], w0.y, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[0][2], w0.z, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[1][0], w0.w, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[1][1], w1.x, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[1][2], w1.y, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[2][0], w1.z, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[2][1], w1.w, acc[r], false);
+      acc[r] = __builtin_amdgcn_sdot4((int)a[2][2], w2, acc[r], false);
+    }
+    unsigned p = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int n = 4 * n4 + r;
+      const bn_t kk = (MODE == EPI_BN) ? k_l[n] : (bn_t)0, ll = (MODE == EPI_BN) ? lam_l[n] : (bn_t)0;
+      p |= (unsigned)requant<MODE>(acc[r], kk, ll, e.mult, e.shift) << (8 * r);
+    }
+    packed[n4] = p;
+  }
+  uint8_t *o = (uint8_t *)g.out + (long long)m * g.N;
+  if (g.vec_store) {
+    // N == NCH and 16-byte aligned rows: one copy of the store code per cache policy
+    auto put = [&](auto nt) {
+      constexpr bool NT = decltype(nt)::value;
+#pragma unroll
+      for (int q = 0; q < NCH / 16; q++)
+        store16<NT>(o + 16 * q, (v4i){(int)packed[4 * q], (int)packed[4 * q + 1], (int)packed[4 * q + 2], (int)packed[4 * q + 3]});
+    };
+    if (g.nt) put(std::true_type{});
+    else put(std::false_type{});
+  } else {
+#pragma unroll
+    for (int n = 0; n < NCH; n++)
+      if (n < g.N) o[n] = (uint8_t)(packed[n >> 2] >> (8 * (n & 3)));
+  }
+}

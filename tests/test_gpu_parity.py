@@ -27,6 +27,9 @@ CONV_GEOMS = [
     (2, 8, 9, 2, 24, 3, 3, (1, 1, 1, 1), (1, 1)),       # 18-byte filters, 24 channels (byte stores)
     (1, 6, 5, 2, 5, 1, 2, (0, 0, 0, 0), (1, 1)),        # 4-byte filters, 5 channels
     (2, 8, 8, 4, 40, 3, 3, (1, 1, 1, 1), (1, 1)),       # 36-byte filters: just past the direct kernel
+    (2, 8, 9, 4, 20, 3, 3, (1, 1, 1, 1), (1, 1)),       # 12-byte filter rows (RGBA stem), row-gather kernel
+    (2, 9, 11, 1, 8, 3, 3, (1, 1, 1, 1), (2, 1)),       # 3-byte filter rows, every alignment of a row start
+    (1, 7, 8, 3, 12, 2, 3, (0, 1, 2, 0), (1, 1)),       # two filter rows, two columns of left padding
 ]
 FLAGS = [(1, 1), (1, 0), (0, 0), (0, 1), (2, 0)]
 
