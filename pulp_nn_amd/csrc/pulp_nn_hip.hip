@@ -237,6 +237,9 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   int blocks = num_cus();
   const int need = (g.units + 2 * nw - 1) / (2 * nw);
   if (blocks > need) blocks = need;
+  // a launch that would leave more than half of the CUs without a workgroup is better off tiled:
+  // every CU takes part there, and staging the weights per workgroup no longer pays
+  if (2 * need < num_cus()) return false;
   dim3 grid(blocks);
   if (tn == 1) launch_pw_stream_ks<1, 1>(mode, ks, wide, g, e, grid, lds, s);
   else if (tn == 2) launch_pw_stream_ks<2, 1>(mode, ks, wide, g, e, grid, lds, s);

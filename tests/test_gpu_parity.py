@@ -83,13 +83,18 @@ PW_GEOMS = [
     (2, 4, 4, 512, 512),
     (1, 9, 11, 3, 100),
     (5, 3, 3, 70, 64),
-    # shapes that take the weights-stationary streaming kernel (>= 2048 pixels, K, N <= 256)
+    # a few thousand pixels with K, N <= 256: tiled kernel, every tile shape
     (4, 32, 32, 16, 32),     # 16 -> 32 channels (MobileNet block 1), K < 64
     (3, 30, 30, 32, 16),     # N = 16
-    (2, 40, 40, 64, 64),     # one channel group
-    (2, 33, 35, 64, 128),    # two channel groups, pixel count not a multiple of 64
+    (2, 40, 40, 64, 64),
+    (2, 33, 35, 64, 128),    # pixel count not a multiple of 64
+    # shapes that take the weights-stationary streaming kernel (>= 32768 pixels, K, N <= 256)
     (16, 112, 112, 32, 64),  # 200704 pixels: the 16-wave shape of the streaming kernel, one channel group
     (16, 112, 113, 16, 32),  # ... 32 channels, pixel count not a multiple of 16 per wave
+    (8, 64, 64, 64, 128),    # two channel groups
+    (8, 64, 65, 128, 256),   # config 1 channels, pixel count not a multiple of 64
+    (9, 64, 64, 192, 192),   # K = 192: four K slices, three channel groups
+    (8, 64, 66, 256, 16),    # K = 256, N = 16
     (16, 65, 64, 64, 300),   # 66560 pixels x 300 channels: the 256 x 256 tiles of the tiled kernel, channel tail
     (2, 33, 33, 256, 200),   # K = 256, channel tail inside the last group
     (2, 40, 30, 48, 100),    # K and N not multiples of 64
