@@ -88,6 +88,36 @@ def test_config3_mobilenet_batch256():
     check_digest("cfg3_b256_logits", got)
 
 
+def test_config3_chain_in_a_hip_graph():
+    """The library allocates nothing, clears nothing and queues on the stream it is given, so a
+    caller can capture the whole chain in a HIP graph.  Replays, with eager work and
+    synchronisations between them, must all reproduce the eager logits."""
+    net = mobilenet.build(256)
+    L = nn(32)
+    runner = mobilenet.Runner(L, net)
+    x = torch.from_numpy(net["x"]).cuda()
+    eager = runner.run(x).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        L.use_torch_stream()
+        runner.run(x)
+    L.use_torch_stream()
+    try:
+        for i in range(3):
+            runner.logits.fill_(-1)
+            for a in runner.act:
+                a.random_(0, 255)      # eager work between the replays; every activation is rewritten by the graph
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert bool((runner.logits == eager).all()), "replay %d differs from the eager run" % i
+    finally:
+        L.set_batch(1)
+
+
 def test_config4_bn64_chain_batch64():
     c = workloads.config4(64, relu=1)
     y = conv(c["x"], c["w"], c["bias"], c["k"], c["lam"], 0, c["out_shift"], c["pads"], c["strides"], 1, 1, 64,
