@@ -22,6 +22,8 @@
 //      "4 pixels of my channel" into "4 channels of one pixel", so that 16
 //      quads write 64 contiguous bytes of an HWC pixel.
 #pragma once
+#include <type_traits>
+
 #include "memops.h"
 #include "requant.h"
 
@@ -483,6 +485,98 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
       else dw3x3_column<S, PL, MODE, FULL, false, false>(col);
     }
   }
+}
+
+// 3x3 depthwise on small square planes (8x8 or 4x4 input, padding 1): a lane keeps the whole
+// plane of its channel in registers (64 or 16 bytes, 16-byte loads; the planes of consecutive
+// channels are contiguous in a CHW image, so a wave reads one contiguous 4 KB / 1 KB run) and
+// works through all its output pixels with the same v_dot4 windows, requantisation and quad
+// transpose as dw3x3_column.  No LDS, no barrier, one wave per workgroup: such a layer is a few
+// MB at batch 256, and with the staged kernel its time goes into launching eight waves per
+// 64-channel tile (about 100 workgroups per microsecond) and into the latency chain load ->
+// LDS -> barrier -> arithmetic of each of them.
+// A filter row that falls outside the plane contributes -128 * (sum of its weights) to every
+// output (activations are held as a - 128, and a = 0 there), added as one constant.
+template <int HW, int S, int MODE>
+__global__ __launch_bounds__(64) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
+{
+  constexpr int RD = HW / 4;                  // dwords per row
+  constexpr int HO = (HW - 1) / S + 1;        // output rows and columns
+  constexpr int XG = HO / 4;                  // groups of 4 output columns
+  constexpr int O0 = 3;                       // byte offset of column -1 in a span that starts one dword left of the group
+  constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
+  static_assert(HW % 4 == 0 && HO % 4 == 0, "whole dwords in, whole groups of 4 columns out");
+  const int lane = threadIdx.x;
+  const int cg = blockIdx.x % g.cgroups, b = blockIdx.x / g.cgroups;
+  const int ch = cg * DW_CG + lane;           // CH % 64 == 0
+
+  unsigned row[HW][RD];
+  {
+    const uint8_t *src = g.in + ((long long)b * g.CH + ch) * (HW * HW);
+#pragma unroll
+    for (int q = 0; q < HW * RD / 4; q++) {
+      const v4i v = *(const v4i *)(src + 16 * q);
+#pragma unroll
+      for (int j = 0; j < 4; j++) row[(4 * q + j) / RD][(4 * q + j) % RD] = (unsigned)v[j] ^ 0x80808080u;
+    }
+  }
+  unsigned wA[3], wB[3];
+  int pad[3], wsum = 0;
+#pragma unroll
+  for (int i = 0; i < 3; i++) {
+    const int8_t *p = g.wt + (long long)ch * 9 + 3 * i;
+    const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
+    wA[i] = k0 | (k1 << 8) | (k2 << 16);
+    wB[i] = wA[i] << 8;
+    const int rs = (int)p[0] + (int)p[1] + (int)p[2];
+    pad[i] = -128 * rs;
+    wsum += rs;
+  }
+  const int corr = 128 * wsum + (g.bias ? (int)g.bias[ch] : 0);
+  bn_t kk = 0, ll = 0;
+  if (MODE == EPI_BN) {
+    kk = e.k[ch];
+    ll = e.lambda[ch];
+  }
+  const bool fastq = (MODE == EPI_BN) ? __all(bn_k_small(kk)) : (e.shift >= 16);
+  const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
+  // after the quad transpose this lane holds 4 consecutive channels of pixel column 4*xg + lane%4
+  uint8_t *obase = g.out + ((long long)b * HO * HO + (lane & 3)) * g.CH + cg * DW_CG + (lane & ~3);
+
+  auto body = [&](auto fq) {
+    constexpr bool FASTQ = decltype(fq)::value;
+#pragma unroll
+    for (int oy = 0; oy < HO; oy++) {
+#pragma unroll
+      for (int xg = 0; xg < XG; xg++) {
+        int acc[4] = {corr, corr, corr, corr};
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+          const int iy = oy * S - 1 + i;
+          if (iy < 0 || iy >= HW) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] += pad[i];
+          } else {
+            unsigned span[NS];
+#pragma unroll
+            for (int d = 0; d < NS; d++) {
+              const int col = xg * S - 1 + d;  // dword column
+              span[d] = (col >= 0 && col < RD) ? row[iy][col < 0 ? 0 : (col >= RD ? RD - 1 : col)] : 0x80808080u;
+            }
+            dw_tap<O0, NS>(span, wA[i], wB[i], acc[0]);
+            dw_tap<O0 + S, NS>(span, wA[i], wB[i], acc[1]);
+            dw_tap<O0 + 2 * S, NS>(span, wA[i], wB[i], acc[2]);
+            dw_tap<O0 + 3 * S, NS>(span, wA[i], wB[i], acc[3]);
+          }
+        }
+        unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], kk, ll, e.mult, e.shift);
+        packed = quad_transpose4x4_perm(packed, sel1, sel2);
+        *(unsigned *)(obase + (long long)(oy * HO + 4 * xg) * g.CH) = packed;
+      }
+    }
+  };
+  if (fastq) body(std::true_type{});
+  else body(std::false_type{});
 }
 
 // Any kernel size / stride / padding: one output per lane per step, one LDS

@@ -442,7 +442,24 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     default: hipLaunchKernelGGL((KERNEL<EPI_RAW>), grid, block, lds, g_stream, g, e); break;        \
   }
 #define DW3(S, PL, M) dw3x3_kernel<S, PL, M>
-  if (lin) {
+  // small square planes, padding 1: one plane per lane, in registers
+  const int ho_plane = (H - 1) / sx + 1;
+  const bool plane = fast && W == H && pt == 1 && pl == 1 && ((H == 8) || (H == 4 && sx == 1)) && Ho == ho_plane &&
+                     Wo == ho_plane && CH % DW_CG == 0 && aligned(in, 16) && aligned(out, 4) &&
+                     (long long)g.B * g.cgroups <= 0x7fffffffLL;
+  if (plane) {
+    const dim3 pgrid((unsigned)(g.B * g.cgroups)), pblock(64);
+#define DWP_MODE(HW, S)                                                                                       \
+  switch (mode) {                                                                                             \
+    case EPI_BN: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_BN>), pgrid, pblock, 0, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_MULT>), pgrid, pblock, 0, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_RAW>), pgrid, pblock, 0, g_stream, g, e); break;        \
+  }
+    if (H == 8 && sx == 1) { DWP_MODE(8, 1) }
+    else if (H == 8) { DWP_MODE(8, 2) }
+    else { DWP_MODE(4, 1) }
+#undef DWP_MODE
+  } else if (lin) {
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
     const dim3 block(64 * DW_WAVES);

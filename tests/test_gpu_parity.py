@@ -147,6 +147,10 @@ DW_GEOMS = [
     (3, 16, 20, 16, 3, 3, (1, 1, 1, 1), (2, 2)),     # ... with a partly filled last group of images
     (5, 32, 12, 24, 3, 3, (1, 1, 1, 1), (2, 2)),     # 32 channels: two images per workgroup, odd batch
     (9, 8, 18, 20, 3, 3, (0, 0, 0, 0), (1, 1)),      # 8 channels: eight images per workgroup, no padding
+    (3, 64, 8, 8, 3, 3, (1, 1, 1, 1), (1, 1)),       # 8x8 planes: one plane per lane, in registers
+    (2, 128, 8, 8, 3, 3, (1, 1, 1, 1), (2, 2)),      # ... stride 2
+    (2, 64, 8, 8, 3, 3, (1, 0, 1, 0), (2, 2)),       # ... stride 2 without bottom / right padding (same output size)
+    (5, 192, 4, 4, 3, 3, (1, 1, 1, 1), (1, 1)),      # 4x4 planes
 ]
 
 
