@@ -250,7 +250,8 @@ def main():
                      wall, dev, np.array_equal(lout.cpu().numpy(), want))
         del xs4, outs4, pooled
 
-        # configuration 3: the whole MobileNetV1-0.5 chain at batch 256 (29 layer launches + 13 layout changes)
+        # configuration 3: the whole MobileNetV1-0.5 chain at batch 256: 29 launches, the layout change
+        # in front of every depthwise layer fused into it (pulp_nn_hip_depthwise_hwc)
         from pulp_nn_amd import mobilenet
         net = mobilenet.build(256)
         runner = mobilenet.Runner(libs[32], net)

@@ -58,6 +58,21 @@ void pulp_nn_hip_hwc_to_chw(const unsigned char *in_hwc, unsigned char *out_chw,
                             unsigned dim_x, unsigned dim_y, unsigned ch,
                             unsigned pad_top, unsigned pad_bottom);
 
+/* The glue above fused into the layer that follows it: a 3x3 depthwise convolution with
+ * padding 1 on all sides and stride 1 or 2 that reads its input as HWC (the output of the
+ * previous conv / pointwise layer) and writes HWC.  Arithmetic and the remaining arguments are
+ * those of pulp_nn_depthwise_generic (k, lambda: int32_t or int64_t arrays as the build
+ * expects; out_shift is taken as int8_t).  Available where the library keeps the rows of a
+ * plane in registers: 8x8 and 4x4 (stride 1) images with a multiple of 64 channels, and
+ * images 16, 32 or 64 pixels wide with a multiple of 4 channels and batch x channels a
+ * multiple of 64.  Any other geometry sets PULP_NN_HIP_ERR_UNSUPPORTED and queues nothing:
+ * call pulp_nn_hip_hwc_to_chw and pulp_nn_depthwise_generic instead. */
+void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bias, unsigned char *Im_out,
+                               const signed char *wt, void *k, void *lambda, unsigned short out_mult,
+                               unsigned short out_shift, unsigned short dim_im_in_x, unsigned short dim_im_in_y,
+                               unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
+                               unsigned short stride, signed char flag_relu, signed char flag_batch_norm);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,6 +82,8 @@ class PulpNN:
         L.pulp_nn_hip_bn_bits.restype = _INT
         L.pulp_nn_hip_hwc_to_chw.argtypes = [_PTR, _PTR] + [C.c_uint] * 5
         L.pulp_nn_hip_hwc_to_chw.restype = None
+        L.pulp_nn_hip_depthwise_hwc.argtypes = [_PTR] * 6 + [_U16] * 8 + [_I8, _I8]
+        L.pulp_nn_hip_depthwise_hwc.restype = None
         assert L.pulp_nn_hip_bn_bits() == bn_bits
 
     # -- added entry points ------------------------------------------------
@@ -127,6 +129,13 @@ class PulpNN:
 
     def hwc_to_chw(self, x, out, dim_x, dim_y, ch, pad_top=0, pad_bottom=0):
         self._call("pulp_nn_hip_hwc_to_chw", _ptr(x), _ptr(out), dim_x, dim_y, ch, pad_top, pad_bottom)
+
+    def depthwise_hwc(self, x, bias, out, wt, k, lam, out_mult, out_shift, dim_in_x, dim_in_y, ch, dim_out_x,
+                      dim_out_y, stride, flag_relu, flag_batch_norm):
+        """3x3 depthwise, padding 1, HWC in and out (the layout change fused in).  Raises
+        PulpNNError (unsupported) for geometries without a fused kernel."""
+        self._call("pulp_nn_hip_depthwise_hwc", _ptr(x), _ptr(bias), _ptr(out), _ptr(wt), _ptr(k), _ptr(lam), out_mult,
+                   out_shift, dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, stride, flag_relu, flag_batch_norm)
 
     # -- the reference API ---------------------------------------------------
     def _conv(self, name, pIn, pIm2Col, bias, pOut, pWeight, k, lam, *scalars):

@@ -487,18 +487,22 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
   }
 }
 
+#define DW_REG_WAVES 4  // waves per workgroup of the register-resident kernels (independent of each other)
+
 // 3x3 depthwise on small square planes (8x8 or 4x4 input, padding 1): a lane keeps the whole
 // plane of its channel in registers (64 or 16 bytes, 16-byte loads; the planes of consecutive
 // channels are contiguous in a CHW image, so a wave reads one contiguous 4 KB / 1 KB run) and
 // works through all its output pixels with the same v_dot4 windows, requantisation and quad
-// transpose as dw3x3_column.  No LDS, no barrier, one wave per workgroup: such a layer is a few
+// transpose as dw3x3_column.  No LDS, no barrier, waves independent: such a layer is a few
 // MB at batch 256, and with the staged kernel its time goes into launching eight waves per
 // 64-channel tile (about 100 workgroups per microsecond) and into the latency chain load ->
 // LDS -> barrier -> arithmetic of each of them.
 // A filter row that falls outside the plane contributes -128 * (sum of its weights) to every
 // output (activations are held as a - 128, and a = 0 there), added as one constant.
-template <int HW, int S, int MODE>
-__global__ __launch_bounds__(64) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
+// HWC: the input is HWC (the layout glue fused in): a lane quad loads a dword (its four channels)
+// of four neighbouring pixels each and transposes it into four pixels of each lane's channel.
+template <int HW, int S, int MODE, bool HWC>
+__global__ __launch_bounds__(64 * DW_REG_WAVES) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
 {
   constexpr int RD = HW / 4;                  // dwords per row
   constexpr int HO = (HW - 1) / S + 1;        // output rows and columns
@@ -506,12 +510,27 @@ __global__ __launch_bounds__(64) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
   constexpr int O0 = 3;                       // byte offset of column -1 in a span that starts one dword left of the group
   constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
   static_assert(HW % 4 == 0 && HO % 4 == 0, "whole dwords in, whole groups of 4 columns out");
-  const int lane = threadIdx.x;
-  const int cg = blockIdx.x % g.cgroups, b = blockIdx.x / g.cgroups;
+  // the waves of a workgroup are independent work items (workgroups of one wave are dispatched
+  // too slowly for a kernel of a few microseconds)
+  const int lane = threadIdx.x & 63;
+  const long long item = (long long)blockIdx.x * DW_REG_WAVES + (threadIdx.x >> 6);
+  if (item >= (long long)g.B * g.cgroups) return;
+  const int cg = (int)(item % g.cgroups), b = (int)(item / g.cgroups);
   const int ch = cg * DW_CG + lane;           // CH % 64 == 0
 
+  const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
   unsigned row[HW][RD];
-  {
+  if constexpr (HWC) {
+    const uint8_t *src = g.in + ((long long)b * (HW * HW) + (lane & 3)) * g.CH + (ch & ~3);
+#pragma unroll
+    for (int y = 0; y < HW; y++)
+#pragma unroll
+      for (int d = 0; d < RD; d++) row[y][d] = *(const unsigned *)(src + (long long)(y * HW + 4 * d) * g.CH);
+#pragma unroll
+    for (int y = 0; y < HW; y++)
+#pragma unroll
+      for (int d = 0; d < RD; d++) row[y][d] = quad_transpose4x4_perm(row[y][d], sel1, sel2) ^ 0x80808080u;
+  } else {
     const uint8_t *src = g.in + ((long long)b * g.CH + ch) * (HW * HW);
 #pragma unroll
     for (int q = 0; q < HW * RD / 4; q++) {
@@ -539,7 +558,6 @@ __global__ __launch_bounds__(64) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
     ll = e.lambda[ch];
   }
   const bool fastq = (MODE == EPI_BN) ? __all(bn_k_small(kk)) : (e.shift >= 16);
-  const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
   // after the quad transpose this lane holds 4 consecutive channels of pixel column 4*xg + lane%4
   uint8_t *obase = g.out + ((long long)b * HO * HO + (lane & 3)) * g.CH + cg * DW_CG + (lane & ~3);
 
@@ -572,6 +590,116 @@ __global__ __launch_bounds__(64) void dw3x3_plane_kernel(DwGeom g, EpiArgs e)
         unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], kk, ll, e.mult, e.shift);
         packed = quad_transpose4x4_perm(packed, sel1, sel2);
         *(unsigned *)(obase + (long long)(oy * HO + 4 * xg) * g.CH) = packed;
+      }
+    }
+  };
+  if (fastq) body(std::true_type{});
+  else body(std::false_type{});
+}
+
+// The same for planes with rows of 16, 32 or 64 bytes (padding 1): a lane keeps the (R-1)*S + 3
+// input rows behind R output rows of its plane in registers, a workgroup (one wave) takes 64
+// consecutive planes of the batch (B * CH planes lie back to back; CH % 4 == 0 keeps the four
+// channels that a lane quad transposes inside one image) and one segment of R output rows.
+// Rows above and below the plane are loaded from a valid address and replaced by zero
+// activations.
+template <int WB, int R, int S, int MODE, bool HWC>
+__global__ __launch_bounds__(64 * DW_REG_WAVES) void dw3x3_rows_kernel(DwGeom g, EpiArgs e)
+{
+  constexpr int RD = WB / 4;                  // dwords per row
+  constexpr int WO = (WB - 1) / S + 1;        // output columns
+  constexpr int XG = WO / 4;                  // groups of 4 output columns
+  constexpr int NIN = (R - 1) * S + 3;        // input rows behind R output rows
+  constexpr int O0 = 3;
+  constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
+  static_assert(WB % 16 == 0 && WO % 4 == 0, "whole 16-byte pieces in, whole groups of 4 columns out");
+  const int lane = threadIdx.x & 63;
+  const int nseg = (g.Ho + R - 1) / R;
+  const long long item = (long long)blockIdx.x * DW_REG_WAVES + (threadIdx.x >> 6);  // one per wave
+  if (item >= g.planes / DW_CG * nseg) return;
+  const int seg = (int)(item % nseg);
+  const long long P = item / nseg * DW_CG + lane;  // plane: image P / CHR, channel P % CHR
+  const int b = (int)(P / g.CHR), ch = (int)(P % g.CHR);
+  const int oy0 = seg * R;
+
+  const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
+  unsigned row[NIN][RD];
+  if constexpr (HWC) {
+    const uint8_t *src = g.in + ((long long)b * g.H * WB + (lane & 3)) * g.CHR + (ch & ~3);
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+      const int iy = oy0 * S - 1 + r;
+      const bool ok = (unsigned)iy < (unsigned)g.H;
+      const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB * g.CHR;
+#pragma unroll
+      for (int d = 0; d < RD; d++) {
+        const unsigned v = *(const unsigned *)(rp + (long long)(4 * d) * g.CHR);
+        row[r][d] = ok ? v : 0u;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < NIN; r++)
+#pragma unroll
+      for (int d = 0; d < RD; d++) row[r][d] = quad_transpose4x4_perm(row[r][d], sel1, sel2) ^ 0x80808080u;
+  } else {
+    const uint8_t *src = g.in + P * ((long long)g.H * WB);
+#pragma unroll
+    for (int r = 0; r < NIN; r++) {
+      const int iy = oy0 * S - 1 + r;
+      const bool ok = (unsigned)iy < (unsigned)g.H;
+      const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB;
+#pragma unroll
+      for (int q = 0; q < RD / 4; q++) {
+        const v4i v = *(const v4i *)(rp + 16 * q);
+#pragma unroll
+        for (int j = 0; j < 4; j++) row[r][4 * q + j] = (ok ? (unsigned)v[j] : 0u) ^ 0x80808080u;
+      }
+    }
+  }
+  unsigned wA[3], wB[3];
+  int wsum = 0;
+#pragma unroll
+  for (int i = 0; i < 3; i++) {
+    const int8_t *p = g.wt + (long long)ch * 9 + 3 * i;
+    const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
+    wA[i] = k0 | (k1 << 8) | (k2 << 16);
+    wB[i] = wA[i] << 8;
+    wsum += (int)p[0] + (int)p[1] + (int)p[2];
+  }
+  const int corr = 128 * wsum + (g.bias ? (int)g.bias[ch] : 0);
+  bn_t kk = 0, ll = 0;
+  if (MODE == EPI_BN) {
+    kk = e.k[ch];
+    ll = e.lambda[ch];
+  }
+  const bool fastq = (MODE == EPI_BN) ? __all(bn_k_small(kk)) : (e.shift >= 16);
+  // after the quad transpose this lane holds the 4 channels of its quad for pixel column 4*xg + lane%4
+  uint8_t *obase = g.out + (((long long)b * g.Ho + oy0) * WO + (lane & 3)) * g.CHR + (ch & ~3);
+
+  auto body = [&](auto fq) {
+    constexpr bool FASTQ = decltype(fq)::value;
+#pragma unroll
+    for (int ro = 0; ro < R; ro++) {
+      if (oy0 + ro >= g.Ho) break;  // (the same for all lanes)
+#pragma unroll
+      for (int xg = 0; xg < XG; xg++) {
+        int acc[4] = {corr, corr, corr, corr};
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+          unsigned span[NS];
+#pragma unroll
+          for (int d = 0; d < NS; d++) {
+            const int col = xg * S - 1 + d;  // dword column
+            span[d] = (col >= 0 && col < RD) ? row[ro * S + i][col < 0 ? 0 : (col >= RD ? RD - 1 : col)] : 0x80808080u;
+          }
+          dw_tap<O0, NS>(span, wA[i], wB[i], acc[0]);
+          dw_tap<O0 + S, NS>(span, wA[i], wB[i], acc[1]);
+          dw_tap<O0 + 2 * S, NS>(span, wA[i], wB[i], acc[2]);
+          dw_tap<O0 + 3 * S, NS>(span, wA[i], wB[i], acc[3]);
+        }
+        unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], kk, ll, e.mult, e.shift);
+        packed = quad_transpose4x4_perm(packed, sel1, sel2);
+        *(unsigned *)(obase + (long long)(ro * WO + 4 * xg) * g.CHR) = packed;
       }
     }
   };

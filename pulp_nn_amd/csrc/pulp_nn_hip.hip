@@ -359,7 +359,7 @@ void linear_common(const char *fn, int mode, const uint8_t *in, const int8_t *bi
 
 void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uint8_t *out, const int8_t *wt,
                       bn_t *k, bn_t *lambda, uint16_t out_mult, int out_shift, int W, int H, int Wo, int Ho, int CH,
-                      int kx, int ky, int pt, int pl, int sx, int sy, int mode)
+                      int kx, int ky, int pt, int pl, int sx, int sy, int mode, bool hwc_in = false)
 {
   if (!in || !out || !wt) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null activation or weight pointer");
   if (W <= 0 || H <= 0 || Wo <= 0 || Ho <= 0 || CH <= 0 || kx <= 0 || ky <= 0 || sx <= 0 || sy <= 0)
@@ -445,20 +445,56 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   // small square planes, padding 1: one plane per lane, in registers
   const int ho_plane = (H - 1) / sx + 1;
   const bool plane = fast && W == H && pt == 1 && pl == 1 && ((H == 8) || (H == 4 && sx == 1)) && Ho == ho_plane &&
-                     Wo == ho_plane && CH % DW_CG == 0 && aligned(in, 16) && aligned(out, 4) &&
+                     Wo == ho_plane && CH % DW_CG == 0 && aligned(in, hwc_in ? 4 : 16) && aligned(out, 4) &&
                      (long long)g.B * g.cgroups <= 0x7fffffffLL;
+  // rows of 16, 32 or 64 bytes, padding 1, any height: a few rows of a plane per lane, in registers
+  const bool rowsk = !plane && fast && pt == 1 && pl == 1 && (W == 16 || W == 32 || W == 64) && Wo == (W - 1) / sx + 1 &&
+                     Ho <= (H - 1) / sy + 1 && CH % 4 == 0 && ((long long)g_batch * CH) % DW_CG == 0 && aligned(in, hwc_in ? 4 : 16) &&
+                     aligned(out, 4) && (long long)g_batch * CH / DW_CG * Ho < 0x7fffffffLL;
+  if (hwc_in && !plane && !rowsk)
+    return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "no fused kernel for this geometry: use pulp_nn_hip_hwc_to_chw and the CHW entry point");
   if (plane) {
-    const dim3 pgrid((unsigned)(g.B * g.cgroups)), pblock(64);
-#define DWP_MODE(HW, S)                                                                                       \
-  switch (mode) {                                                                                             \
-    case EPI_BN: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_BN>), pgrid, pblock, 0, g_stream, g, e); break;     \
-    case EPI_MULT: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_MULT>), pgrid, pblock, 0, g_stream, g, e); break; \
-    default: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_RAW>), pgrid, pblock, 0, g_stream, g, e); break;        \
+    const dim3 pgrid((unsigned)(((long long)g.B * g.cgroups + DW_REG_WAVES - 1) / DW_REG_WAVES)), pblock(64 * DW_REG_WAVES);
+#define DWP_LAYOUT(HW, S, HWC)                                                                                            \
+  switch (mode) {                                                                                                         \
+    case EPI_BN: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_BN, HWC>), pgrid, pblock, 0, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_MULT, HWC>), pgrid, pblock, 0, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((dw3x3_plane_kernel<HW, S, EPI_RAW, HWC>), pgrid, pblock, 0, g_stream, g, e); break;        \
   }
+#define DWP_MODE(HW, S)                      \
+  if (hwc_in) { DWP_LAYOUT(HW, S, true) }    \
+  else { DWP_LAYOUT(HW, S, false) }
     if (H == 8 && sx == 1) { DWP_MODE(8, 1) }
     else if (H == 8) { DWP_MODE(8, 2) }
     else { DWP_MODE(4, 1) }
 #undef DWP_MODE
+#undef DWP_LAYOUT
+  } else if (rowsk) {
+    const long long groups = (long long)g_batch * CH / DW_CG;
+#define DWR_LAYOUT(WB, R, S, HWC)                                                                                                \
+  {                                                                                                                              \
+    const dim3 rgrid((unsigned)((groups * ((Ho + R - 1) / R) + DW_REG_WAVES - 1) / DW_REG_WAVES)), rblock(64 * DW_REG_WAVES);    \
+    switch (mode) {                                                                                                              \
+      case EPI_BN: hipLaunchKernelGGL((dw3x3_rows_kernel<WB, R, S, EPI_BN, HWC>), rgrid, rblock, 0, g_stream, g, e); break;      \
+      case EPI_MULT: hipLaunchKernelGGL((dw3x3_rows_kernel<WB, R, S, EPI_MULT, HWC>), rgrid, rblock, 0, g_stream, g, e); break;  \
+      default: hipLaunchKernelGGL((dw3x3_rows_kernel<WB, R, S, EPI_RAW, HWC>), rgrid, rblock, 0, g_stream, g, e); break;         \
+    }                                                                                                                            \
+  }
+#define DWR_MODE(WB, R, S)                       \
+  {                                              \
+    if (hwc_in) DWR_LAYOUT(WB, R, S, true)       \
+    else DWR_LAYOUT(WB, R, S, false)             \
+  }
+    g.CHR = CH;
+    g.planes = (long long)g_batch * CH;
+    if (W == 16 && sx == 1) DWR_MODE(16, 8, 1)
+    else if (W == 16) DWR_MODE(16, 4, 2)
+    else if (W == 32 && sx == 1) DWR_MODE(32, 4, 1)
+    else if (W == 32) DWR_MODE(32, 4, 2)
+    else if (sx == 1) DWR_MODE(64, 2, 1)
+    else DWR_MODE(64, 2, 2)
+#undef DWR_MODE
+#undef DWR_LAYOUT
   } else if (lin) {
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
@@ -737,6 +773,17 @@ void pulp_nn_add(uint8_t *Im_in_1, uint8_t *Im_in_2, uint8_t *Im_out, uint16_t o
 
 DW_FORWARD(pulp_nn_depthwise_generic)
 DW_FORWARD(pulp_nn_depthwise_generic_less_4_weights)
+
+void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bias, unsigned char *Im_out,
+                               const signed char *wt, void *k, void *lambda, unsigned short out_mult,
+                               unsigned short out_shift, unsigned short dim_im_in_x, unsigned short dim_im_in_y,
+                               unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
+                               unsigned short stride, signed char flag_relu, signed char flag_batch_norm)
+{
+  depthwise_common(__func__, Im_in, (const int8_t *)bias, Im_out, (const int8_t *)wt, (bn_t *)k, (bn_t *)lambda, out_mult,
+                   out_shift, dim_im_in_x, dim_im_in_y, dim_im_out_x, dim_im_out_y, ch, 3, 3, 1, 1, stride, stride,
+                   epi_mode(flag_relu, flag_batch_norm, true), true);
+}
 
 void pulp_nn_depthwise_3x3_s1(uint8_t *In_Img, uint8_t *Out_Img, int R, int C, int CH, int p_l, int p_r,
                               int8_t *Kernel, int8_t out_shift, uint16_t out_mult, bn_t *kappa, bn_t *lambda,

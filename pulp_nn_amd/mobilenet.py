@@ -4,7 +4,8 @@ average pooling and a 512 -> 1000 linear layer with int32 output.
 
 Everything runs through the C API: pulp_nn_conv_Ho_parallel, pulp_nn_depthwise_generic,
 pulp_nn_pointwise_HoWo_parallel, pulp_nn_avgpool, pulp_nn_linear_out_32, plus
-pulp_nn_hip_hwc_to_chw between a pointwise output (HWC) and the next depthwise input (CHW),
+pulp_nn_hip_hwc_to_chw between a pointwise output (HWC) and the next depthwise input (CHW)
+(or, where the library has a kernel for it, the two fused: pulp_nn_hip_depthwise_hwc),
 a step the reference leaves to the application.
 
 Parameters are seeded like configuration 0 (int8 weights and bias, 32-bit k in [256, 1024],
@@ -17,6 +18,8 @@ import json
 import os
 
 import numpy as np
+
+from .api import PulpNNError
 
 WIDTHS = (32, 64, 64, 128, 128, 256, 256, 256, 256, 256, 256, 512, 512)
 STRIDE2_BLOCKS = (2, 4, 6, 12)   # 1-based
@@ -77,9 +80,13 @@ def build(batch=256, shifts=None):
 class Runner:
     """Uploads the parameters once and runs the chain on the GPU through the C API."""
 
-    def __init__(self, nn, net):
+    def __init__(self, nn, net, fused=True):
         import torch
         self.nn, self.net, self.torch = nn, net, torch
+        # fused: depthwise layers read the HWC output of the previous layer directly
+        # (pulp_nn_hip_depthwise_hwc) where the library has a kernel for it; otherwise, and with
+        # fused=False, the chain is the reference's: pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic
+        self.fused, self.unfused = fused, set()
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
         self.params = [dict(w=dev(L["w"]), bias=dev(L["bias"]), k=dev(L["k"]), lam=dev(L["lam"]))
                        for L in net["layers"]]
@@ -103,6 +110,17 @@ class Runner:
                 nn.pulp_nn_conv_Ho_parallel(cur, None, P["bias"], out, P["w"], P["k"], P["lam"], 0, L["shift"],
                                             hi, hi, ci, ho, ho, co, 3, 3, 1, 1, 1, 1, s, s, 1, 1)
             elif L["kind"] == "dw":
+                if self.fused and i not in self.unfused:
+                    try:
+                        # layout change fused into the depthwise kernel
+                        nn.depthwise_hwc(cur, P["bias"], out, P["w"], P["k"], P["lam"], 0, L["shift"],
+                                         hi, hi, ci, ho, ho, s, 1, 1)
+                        cur = out
+                        continue
+                    except PulpNNError as err:
+                        if err.code != 2:
+                            raise
+                        self.unfused.add(i)   # no fused kernel for this geometry
                 chw = self.chw[i]
                 nn.hwc_to_chw(cur, chw, hi, hi, ci)
                 nn.pulp_nn_depthwise_generic(chw, None, P["bias"], out, P["w"], None, P["k"], P["lam"], 0, L["shift"],

@@ -80,6 +80,22 @@ def depthwise_generic(x, wt, bias, k, lam, mult, shift, pads, strides, relu, bn,
     return out.cpu().numpy()
 
 
+def depthwise_hwc(x_hwc, wt, bias, k, lam, mult, shift, stride, relu, bn, bn_bits=32):
+    """3x3, padding 1, HWC in and out (pulp_nn_hip_depthwise_hwc)."""
+    B, H, W, CH = x_hwc.shape
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+    L = nn(bn_bits)
+    out = torch.full((B, Ho, Wo, CH), 0xA5, dtype=torch.uint8, device="cuda")
+    L.set_batch(B)
+    try:
+        L.depthwise_hwc(dev(x_hwc), dev(bias), out, dev(wt), bn_dev(k, bn_bits), bn_dev(lam, bn_bits), mult, shift,
+                        W, H, CH, Wo, Ho, stride, relu, bn)
+        L.sync()
+    finally:
+        L.set_batch(1)
+    return out.cpu().numpy()
+
+
 def depthwise_3x3_s1(xpad, kern, k, lam, mult, shift, relu, bn, bn_bits=32, p_l=1, p_r=1):
     B, CH, R, Cw = xpad.shape
     L = nn(bn_bits)

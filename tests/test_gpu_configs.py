@@ -86,6 +86,13 @@ def test_config3_mobilenet_batch256():
         assert_same(runner.act[i][:2].cpu().numpy(), w, "config 3 layer %s" % Ld["name"])
     assert_same(got[:2], want_logits, "config 3 logits")
     check_digest("cfg3_b256_logits", got)
+    assert not runner.unfused, "depthwise layers without a fused kernel: %s" % sorted(runner.unfused)
+    # the same chain with the layout changes as separate launches (the reference's call sequence)
+    plain = mobilenet.Runner(L, net, fused=False)
+    got2 = plain.run(x)
+    L.sync()
+    L.set_batch(1)
+    check_digest("cfg3_b256_logits", got2.cpu().numpy())
 
 
 def test_config3_chain_in_a_hip_graph():

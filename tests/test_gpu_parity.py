@@ -5,8 +5,9 @@ import numpy as np
 import pytest
 
 import oracle
-from gpu_helpers import (add, assert_same, avgpool, conv, depthwise_3x3_s1, depthwise_generic, linear,
+from gpu_helpers import (add, assert_same, avgpool, conv, depthwise_3x3_s1, depthwise_generic, depthwise_hwc, linear,
                          linear_out_32, maxpool, nn, rand_s8, rand_u8, rng_for)
+from pulp_nn_amd import PulpNNError
 
 pytestmark = pytest.mark.gpu
 
@@ -151,6 +152,15 @@ DW_GEOMS = [
     (2, 128, 8, 8, 3, 3, (1, 1, 1, 1), (2, 2)),      # ... stride 2
     (2, 64, 8, 8, 3, 3, (1, 0, 1, 0), (2, 2)),       # ... stride 2 without bottom / right padding (same output size)
     (5, 192, 4, 4, 3, 3, (1, 1, 1, 1), (1, 1)),      # 4x4 planes
+    (4, 16, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1)),     # 64-byte rows, a few rows per lane in registers; 16 channels
+    (2, 32, 64, 64, 3, 3, (1, 1, 1, 1), (2, 2)),     # ... stride 2, 32 channels
+    (1, 64, 32, 32, 3, 3, (1, 1, 1, 1), (1, 1)),     # 32-byte rows
+    (2, 64, 32, 32, 3, 3, (1, 1, 1, 1), (2, 2)),
+    (1, 128, 16, 16, 3, 3, (1, 1, 1, 1), (1, 1)),    # 16-byte rows
+    (1, 128, 16, 16, 3, 3, (1, 1, 1, 1), (2, 2)),
+    (1, 64, 11, 16, 3, 3, (1, 1, 1, 1), (1, 1)),     # ... height not a multiple of the rows per lane
+    (2, 32, 9, 32, 3, 3, (1, 1, 1, 1), (2, 2)),      # ... stride 2, odd height
+    (1, 64, 12, 16, 3, 3, (1, 0, 1, 1), (1, 1)),     # ... no bottom padding: one output row fewer
 ]
 
 
@@ -190,6 +200,43 @@ def test_depthwise_3x3_s1(shape, flags, bn_bits):
     want = oracle.depthwise_3x3_s1(xpad, kern, k, lam, 600, shift, 1, 1, relu, bn, bn_bits)
     got = depthwise_3x3_s1(xpad, kern, k, lam, 600, shift, relu, bn, bn_bits)
     assert_same(got, want, "depthwise_3x3_s1")
+
+
+DW_HWC_GEOMS = [
+    # B, CH, H, W, stride: every kernel shape behind pulp_nn_hip_depthwise_hwc
+    (3, 64, 8, 8, 1), (2, 128, 8, 8, 2), (5, 192, 4, 4, 1),
+    (4, 16, 64, 64, 1), (2, 32, 64, 64, 2), (1, 64, 32, 32, 1), (2, 64, 32, 32, 2),
+    (1, 128, 16, 16, 1), (1, 128, 16, 16, 2), (1, 64, 11, 16, 1), (2, 32, 9, 32, 2), (16, 4, 7, 16, 1),
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", FLAGS)
+@pytest.mark.parametrize("geom", DW_HWC_GEOMS, ids=lambda g: "x".join(map(str, g[:4])) + "s%d" % g[4])
+def test_depthwise_hwc(geom, flags, bn_bits):
+    """The fused layout change + depthwise against the oracle's CHW depthwise on the transposed input."""
+    B, CH, H, W, stride = geom
+    relu, bn = flags
+    r = rng_for(3500 + 17 * relu + bn + bn_bits)
+    x_hwc, wt, b = rand_u8(r, (B, H, W, CH)), rand_s8(r, (CH, 3, 3)), rand_s8(r, (CH,))
+    if bn_bits == 32:
+        k, lam, bshift = r.integers(2 ** 12, 2 ** 14 + 1, CH), r.integers(-2 ** 16, 2 ** 16 + 1, CH), 16
+    else:
+        k, lam, bshift = r.integers(2 ** 20, 2 ** 24 + 1, CH), r.integers(-2 ** 36, 2 ** 36 + 1, CH), 28
+    shift = bshift if (relu and bn) else (14 if relu else 6)
+    x_chw = np.ascontiguousarray(x_hwc.transpose(0, 3, 1, 2))
+    want = oracle.depthwise_generic(x_chw, wt, b, k, lam, 900, shift, (1, 1, 1, 1), (stride, stride), relu, bn, bn_bits)
+    got = depthwise_hwc(x_hwc, wt, b, k, lam, 900, shift, stride, relu, bn, bn_bits)
+    assert_same(got, want, "pulp_nn_hip_depthwise_hwc")
+
+
+def test_depthwise_hwc_unsupported_geometry_is_rejected():
+    r = rng_for(3600)
+    x_hwc, wt, b = rand_u8(r, (1, 9, 9, 5)), rand_s8(r, (5, 3, 3)), rand_s8(r, (5,))
+    k, lam = r.integers(2 ** 12, 2 ** 14 + 1, 5), r.integers(-2 ** 16, 2 ** 16 + 1, 5)
+    with pytest.raises(PulpNNError) as ei:
+        depthwise_hwc(x_hwc, wt, b, k, lam, 900, 16, 1, 1, 1, 32)
+    assert ei.value.code == 2
 
 
 @pytest.mark.parametrize("bn_bits", [32, 64])
