@@ -112,6 +112,10 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
   if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
   else
+  // 128 px x 64 ch while 128 x 128 tiles would give a CU at most one workgroup: twice the workgroups to
+  // hide each other's latency (such layers are a few K slices long)
+  if (g.N > 64 && (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) <= num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);
+  else
   if (g.N > 64) launch_igemm_mode<4, 2, 2, GATHER>(mode, g, e, s);       // 128 px x 128 ch
   else if (g.N > 32 && (g.M + 255) / 256 < 2 * num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);  // 128 px x 64 ch: more workgroups
   else if (g.N > 32) launch_igemm_mode<4, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 64 ch
