@@ -47,7 +47,6 @@ struct DwGeom {
   int inc_dw, inc_row, inc_c;
   int in_align4;  // input pointer and W are multiples of 4: aligned dword loads are safe
   int out_vec4;   // output pointer and CH are multiples of 4: dword stores are safe
-  int nt;         // write the output with non-temporal stores
   // Packing of layers with fewer than 64 channels (dw3x3_lin_kernel only): CH and B describe the
   // input re-read as images of 64 planes (CHW images lie back to back, so that is the same memory);
   // CHR is the real channel count, planes the real number of planes B_real * CHR.
@@ -245,7 +244,7 @@ struct DwColumn {
   int store, nbytes;
 };
 
-template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ, bool NT = false>
+template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ>
 __device__ __forceinline__ void dw3x3_column(DwColumn c)
 {
   constexpr int O0 = 4 - PL;
@@ -269,7 +268,7 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
     unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], c.k, c.lambda, c.mult, c.shift);
     packed = quad_transpose4x4_perm(packed, c.sel1, c.sel2);
     if constexpr (FULL) {
-      store4<NT>(c.o, (int)packed);
+      *(unsigned *)c.o = packed;
     } else {
       if (c.store == 0) {
         *(unsigned *)c.o = packed;
@@ -473,11 +472,7 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
     col.store = (4 * xg + (lane & 3) >= g.Wo || left <= 0) ? 2 : ((g.out_vec4 && left >= 4) ? 0 : 1);
     col.nbytes = (int)min(4ll, max(left, 0ll));
     const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
-    if (FULL && fastq && g.nt) {
-      // one more copy of the common case for the streaming store policy
-      if (edge) dw3x3_column<S, PL, MODE, FULL, true, true, FULL>(col);
-      else dw3x3_column<S, PL, MODE, FULL, false, true, FULL>(col);
-    } else if (fastq) {
+    if (fastq) {
       if (edge) dw3x3_column<S, PL, MODE, FULL, true, true>(col);
       else dw3x3_column<S, PL, MODE, FULL, false, true>(col);
     } else {

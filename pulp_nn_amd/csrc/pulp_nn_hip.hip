@@ -436,7 +436,6 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   g.inc_c = carry / g.NR;
   g.in_align4 = aligned(in, 4) && (W % 4 == 0);
   g.out_vec4 = aligned(out, 4) && (CH % 4 == 0);
-  g.nt = g.planes * Ho * Wo >= PULPNN_NT_BYTES;
   const size_t lds = (size_t)DW_CG * g.CSD * 4;
   dim3 grid(g.total), block(256);
 #define DW_LAUNCH(KERNEL)                                                                   \
