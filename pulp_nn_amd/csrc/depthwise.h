@@ -489,9 +489,9 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
 // channels are contiguous in a CHW image, so a wave reads one contiguous 4 KB / 1 KB run) and
 // works through all its output pixels with the same v_dot4 windows, requantisation and quad
 // transpose as dw3x3_column.  No LDS, no barrier, waves independent: such a layer is a few
-// MB at batch 256, and with the staged kernel its time goes into launching eight waves per
-// 64-channel tile (about 100 workgroups per microsecond) and into the latency chain load ->
-// LDS -> barrier -> arithmetic of each of them.
+// MB at batch 256, and with the staged kernel its time goes into the latency chain load ->
+// LDS -> barrier -> arithmetic of a thousand eight-wave workgroups, only part of which are
+// resident at a time.
 // A filter row that falls outside the plane contributes -128 * (sum of its weights) to every
 // output (activations are held as a - 128, and a = 0 there), added as one constant.
 // HWC: the input is HWC (the layout glue fused in): a lane quad loads a dword (its four channels)
@@ -505,8 +505,8 @@ __global__ __launch_bounds__(64 * DW_REG_WAVES) void dw3x3_plane_kernel(DwGeom g
   constexpr int O0 = 3;                       // byte offset of column -1 in a span that starts one dword left of the group
   constexpr int NS = (O0 + 3 * S + 2) / 4 + 1;
   static_assert(HW % 4 == 0 && HO % 4 == 0, "whole dwords in, whole groups of 4 columns out");
-  // the waves of a workgroup are independent work items (workgroups of one wave are dispatched
-  // too slowly for a kernel of a few microseconds)
+  // the waves of a workgroup are independent work items (fewer, larger workgroups start sooner:
+  // this kernel lasts a few microseconds)
   const int lane = threadIdx.x & 63;
   const long long item = (long long)blockIdx.x * DW_REG_WAVES + (threadIdx.x >> 6);
   if (item >= (long long)g.B * g.cgroups) return;
