@@ -7,7 +7,8 @@
 // per-slice latency instead (16 sequential slices for K = 1024).  Here a
 // workgroup of four waves owns 16 output neurons.  The waves split the work by
 // blocks of 64 rows and, when there are fewer than four such blocks, by parts of
-// K as well; a wave fetches the weight fragment (16 rows x 64 bytes) and the
+// K as well (when the neurons alone make too few workgroups for the machine, the row blocks go to
+// separate workgroups and K is always split in four); a wave fetches the weight fragment (16 rows x 64 bytes) and the
 // activation fragments (64 rows x 64 bytes, shared by all workgroups and therefore
 // cache resident) of four K slices at a time straight from global memory in the
 // MFMA operand layout - twenty loads in flight, no staging - and the partial sums
@@ -25,7 +26,7 @@ struct SkinnyGeom {
   const int8_t *bias;  // int8 [N]; int32 [N] for EPI_OUT32; may be null
   void *out;           // [M][N] uint8, or int32 for EPI_OUT32
   int M, N, K;         // M <= 256, K % 16 == 0, 16-byte aligned rows
-  int kparts;          // 4, 2 or 1 parts of K: kparts * ceil(M / 64) <= 4
+  int kparts;          // 4, 2 or 1 parts of K; a workgroup takes 4 / kparts blocks of 64 rows, gridDim.y the rest
 };
 
 template <int MODE>
@@ -37,7 +38,8 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(SkinnyGeom g, EpiArg
   const int l16 = lane & 15, lgrp = lane >> 4;
   const int n0 = blockIdx.x * 16;  // this workgroup's 16 neurons
   const int KT = (g.K + 63) / 64;
-  const int rb = wave / g.kparts, kp = wave % g.kparts;  // block of 64 rows, part of K
+  // block of 64 rows (blockIdx.y counts the row blocks that other workgroups of the same neurons take), part of K
+  const int rb = blockIdx.y * (4 / g.kparts) + wave / g.kparts, kp = wave % g.kparts;
   const int mb = rb * 64;
   const int kt0 = KT * kp / g.kparts, kt1 = KT * (kp + 1) / g.kparts;
   const bool active = mb < g.M;

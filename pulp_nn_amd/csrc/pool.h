@@ -121,11 +121,21 @@ __global__ __launch_bounds__(256) void avgpool_kernel(PoolGeom g, AvgArgs a)
   const int xs = max(0, ox * g.sx - g.pl), xe = min(ox * g.sx - g.pr + g.kx, g.W);
   const uint8_t *img = g.in + (long long)b * g.H * g.W * g.C + c;
   unsigned sum[4] = {0, 0, 0, 0};
+  // four taps at a time, their loads issued together (taps past the window re-read its last
+  // column and are not counted): one load per round trip would make the window size the
+  // kernel's latency
   for (int y = ys; y < ye; y++)
-    for (int x = xs; x < xe; x++) {
-      const unsigned v = load4(img + ((long long)y * g.W + x) * g.C, n, g.vec4);
+    for (int x = xs; x < xe; x += 4) {
+      unsigned v[4];
 #pragma unroll
-      for (int j = 0; j < 4; j++) sum[j] += (v >> (8 * j)) & 0xFF;
+      for (int i = 0; i < 4; i++) v[i] = load4(img + ((long long)y * g.W + min(x + i, xe - 1)) * g.C, n, g.vec4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        if (x + i < xe) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) sum[j] += (v[i] >> (8 * j)) & 0xFF;
+        }
+      }
     }
   const unsigned ksize = (unsigned)(g.kx * g.ky);
   unsigned packed = 0;

@@ -328,9 +328,12 @@ void linear_common(const char *fn, int mode, const uint8_t *in, const int8_t *bi
   if (!dim_vec || !num_o_neurons) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
   // few rows: a workgroup per 16 neurons streams their weights once, no staging and no K-slice barriers
   if (rows <= 256 && dim_vec % 16 == 0 && aligned(in, 16) && aligned(w, 16) && aligned(out, 4)) {
-    const int rblocks = (rows + 63) / 64;
-    SkinnyGeom sg = {in, w, bias, out, rows, (int)num_o_neurons, (int)dim_vec, rblocks == 1 ? 4 : (rblocks == 2 ? 2 : 1)};
-    const dim3 grid((num_o_neurons + 15) / 16), block(256);
+    const int rblocks = (rows + 63) / 64, ngroups = (num_o_neurons + 15) / 16;
+    // K in four parts and a workgroup per block of rows while that still leaves CUs without work
+    const bool spread = ngroups * rblocks <= 2 * num_cus();
+    const int kparts = spread ? 4 : (rblocks == 1 ? 4 : (rblocks == 2 ? 2 : 1));
+    SkinnyGeom sg = {in, w, bias, out, rows, (int)num_o_neurons, (int)dim_vec, kparts};
+    const dim3 grid(ngroups, spread ? rblocks : 1), block(256);
     switch (mode) {
       case EPI_BN: hipLaunchKernelGGL(linear_skinny_kernel<EPI_BN>, grid, block, 0, g_stream, sg, e); break;
       case EPI_MULT: hipLaunchKernelGGL(linear_skinny_kernel<EPI_MULT>, grid, block, 0, g_stream, sg, e); break;
