@@ -121,3 +121,28 @@ def test_random_linear(case, bn_bits):
     want = oracle.linear(x, w, b, k, lam, mult, shift, relu, bn, bn_bits)
     got = linear(x, w, b, k, lam, mult, shift, relu, bn, bn_bits)
     assert_same(got, want, "linear %s" % (case,))
+
+
+def _pw_cases(n, seed):
+    """Pixel counts on both sides of the streaming kernel's threshold, channel counts on and off its list."""
+    r = rng_for(seed)
+    px = [(1, 45, 45), (2, 32, 32), (4, 64, 64), (7, 68, 68), (8, 64, 64), (5, 81, 81), (3, 100, 110)]
+    return [px[int(r.integers(0, len(px)))] + (int(r.choice([16, 48, 64, 128, 200, 256])),
+                                              int(r.choice([16, 32, 64, 100, 128, 192, 256]))) for _ in range(n)]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("case", _pw_cases(20, 9004), ids=lambda c: "x".join(map(str, c)))
+def test_random_pointwise(case, bn_bits):
+    B, H, W, Ci, Co = case
+    r = rng_for(hash(case) % (2 ** 31) + bn_bits)
+    relu, bn = _flags(r)
+    x, w, b = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, 1, 1, Ci)), rand_s8(r, (Co,))
+    k, lam, bshift = _bn(r, Co, bn_bits)
+    lg = int(np.log2(max(Ci, 2) ** 0.5 * 128 * 74))
+    shift = bshift if (relu and bn) else ((lg + 3) if relu == 1 else max(lg - 7, 0))
+    mult = int(r.integers(64, 1025))
+    want = oracle.pointwise(x, w, b, k, lam, mult, shift, relu, bn, bn_bits)
+    got = conv(x, w, b, k, lam, mult, shift, (0, 0, 0, 0), (1, 1), relu, bn, bn_bits, out_hw=(H, W),
+               fn="pulp_nn_pointwise_HoWo_parallel")
+    assert_same(got, want, "pointwise %s" % (case,))
