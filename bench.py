@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA, op/s
 PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
-HBM_TRAFFIC_CFG1 = int((12731.0 * 2.0 + 50188.7) * 1024)   # measured: FETCH_SIZE 12731.0 KiB x 2.0 + WRITE_SIZE 50188.7 KiB
+HBM_TRAFFIC_CFG1 = int((12728.0 * 2.0 + 50193.0) * 1024)   # measured: FETCH_SIZE 12728.0 KiB x 2.0 + WRITE_SIZE 50193.0 KiB
 
 
 def main():
