@@ -319,6 +319,13 @@ def test_avgpool(bn_bits):
             want = oracle.avgpool(x2, kernel, strides, pads, out_hw, lam, sh, ad, rq, bn_bits)
             got = avgpool(x2, kernel, strides, out_hw, pads, lam, sh, ad, rq, bn_bits)
             assert_same(got, want, "avgpool %s %s" % (pads, (rq, lam)))
+    # windows wider than one batch of loads, channel tail
+    x3 = rand_u8(r, (2, 7, 7, 22))
+    for pads, kernel, strides, out_hw in [((0, 0, 0, 0), (7, 7), (7, 7), (1, 1)), ((2, 2, 2, 2), (5, 5), (1, 1), (7, 7)),
+                                          ((0, 0, 0, 0), (6, 5), (1, 2), (2, 2))]:
+        want = oracle.avgpool(x3, kernel, strides, pads, out_hw, 0, 0, 0, 0, bn_bits)
+        got = avgpool(x3, kernel, strides, out_hw, pads, 0, 0, 0, 0, bn_bits)
+        assert_same(got, want, "avgpool %s %s" % (pads, kernel))
 
 
 def test_add():
