@@ -179,6 +179,8 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
     }
   }
 
+  const int KT = (g.K + IGEMM_BK - 1) / IGEMM_BK;
+
   // The loads of K slice kt+1 are in flight while slice kt is multiplied; they are staged
   // into the other LDS buffer afterwards.  (A second register set for a two-slice distance
   // costs 70 registers and with them a workgroup per CU, for no gain: the kernel is bound
@@ -210,13 +212,17 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
         R.w[i] = (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
       }
       R.amask = R.wmask = ~0u;
-      // advance to the next K slice (scalar)
-      u_slice++;
-      u_ci += IGEMM_BK;
-      if (u_ci >= g.Ci) {
-        u_ci = 0;
-        u_tap++;
-        if (++u_fx == g.kx) { u_fx = 0; ++u_fy; }
+      // advance to the next K slice (scalar).  The prefetch runs one slice past the end; that
+      // request repeats the last real slice instead, so no address beyond the caller's buffers is
+      // ever formed (buffer loads do not range-check the scalar offset).
+      if (u_slice + 1 < KT) {
+        u_slice++;
+        u_ci += IGEMM_BK;
+        if (u_ci >= g.Ci) {
+          u_ci = 0;
+          u_tap++;
+          if (++u_fx == g.kx) { u_fx = 0; ++u_fy; }
+        }
       }
       return;
     }
@@ -315,7 +321,6 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   const int wfrag_row0 = wave_n * WN + l16;
   const int afrag_row0 = wave_m * WM + l16;
 
-  const int KT = (g.K + IGEMM_BK - 1) / IGEMM_BK;
   auto compute = [&](int cur) {
     v4i wf[TN], af[TM];
 #pragma unroll

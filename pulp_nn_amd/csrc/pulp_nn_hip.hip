@@ -590,7 +590,11 @@ bool pool_geom(const char *fn, PoolGeom *g, uint8_t *in, uint8_t *out, uint16_t 
 
 extern "C" {
 
-void pulp_nn_hip_set_batch(unsigned n_images) { g_batch = n_images ? n_images : 1; }
+void pulp_nn_hip_set_batch(unsigned n_images)
+{
+  if (n_images > 0x7fffffffu) return set_error(PULP_NN_HIP_ERR_ARGUMENT, __func__, "batch too large");
+  g_batch = n_images ? n_images : 1;
+}
 unsigned pulp_nn_hip_get_batch(void) { return g_batch; }
 void pulp_nn_hip_set_stream(void *hip_stream) { g_stream = (hipStream_t)hip_stream; }
 void *pulp_nn_hip_get_stream(void) { return (void *)g_stream; }

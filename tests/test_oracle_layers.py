@@ -321,6 +321,61 @@ def test_avgpool_padding_arguments_as_written():
             np.testing.assert_array_equal(got[oy, ox], want.astype(np.uint8))
 
 
+def test_avgpool_asymmetric_padding_known_answer():
+    """Hand-derived: 3x3 image, one channel, 2x2 window, stride 1, pads (t,b,l,r) = (0,1,0,1).
+    pulp_nn_avgpool.c:82-86: rows [max(0, iy - padding_b), min(iy - padding_t + 2, 3)),
+    columns [max(0, ix - padding_l), min(ix - padding_r + 2, 3)); divisor 4.
+      in = [[ 4,  8, 12],
+            [16, 20, 24],
+            [28, 32, 36]]
+    output (1,1): rows [0,3), columns [1,2) -> (8+20+32)/4 = 15.  Reading padding_t as the row
+    start and padding_l as the column end would give rows [1,3), columns [1,3) -> 112/4 = 28.
+    output (0,0): rows [0,2), columns [0,1) -> (4+16)/4 = 5   (the other reading: (4+8+16+20)/4 = 12)
+    output (0,1): rows [0,2), columns [1,2) -> (8+20)/4 = 7   (other: 64/4 = 16)
+    output (1,0): rows [0,3), columns [0,1) -> (4+16+28)/4 = 12 (other: 96/4 = 24)"""
+    x = np.array([[4, 8, 12], [16, 20, 24], [28, 32, 36]], np.uint8).reshape(3, 3, 1)
+    got = oracle.avgpool(x, (2, 2), (1, 1), pads=(0, 1, 0, 1), out_hw=(2, 2))
+    np.testing.assert_array_equal(got[:, :, 0], np.array([[5, 7], [12, 15]], np.uint8))
+    # the mirrored pads (1,0,1,0): rows [max(0, iy), min(iy - 1 + 2, 3)), columns [max(0, ix - 1), min(ix + 2, 3))
+    # (0,0): row 0, columns [0,2) -> 12/4 = 3; (0,1): row 0, columns [0,3) -> 24/4 = 6
+    # (1,0): row 1, columns [0,2) -> 36/4 = 9; (1,1): row 1, columns [0,3) -> 60/4 = 15
+    got = oracle.avgpool(x, (2, 2), (1, 1), pads=(1, 0, 1, 0), out_hw=(2, 2))
+    np.testing.assert_array_equal(got[:, :, 0], np.array([[3, 6], [9, 15]], np.uint8))
+
+
+def test_maxpool_padded_known_answers():
+    """Hand-derived from pulp_nn_maxpool.c:58-144.
+    (a) 3x3 window, stride 2, padding 1 on a 5x5 one-channel image: column windows
+        [0,2) (start -1 < 0 -> the target column 0), [1,4), [3,5) (end clamped to 5), rows alike.
+          in = [[ 1,  2,  3,  4,  5],
+                [10,  9,  8,  7,  6],
+                [11, 12, 13, 14, 15],
+                [20, 19, 18, 17, 16],
+                [21, 22, 23, 24, 25]]
+        x pass (per row): [2,4,5] [10,9,7] [12,14,15] [20,19,17] [22,24,25]
+        y pass rows [0,2) [1,4) [3,5): [[10,9,7],[20,19,17],[22,24,25]]
+    (b) the left clamp is the output column itself, not column 0 (:65-68): 1x4 image [9,1,5,3],
+        3-wide window, stride 1, padding_l 2, three outputs.  ix=0: start -2 -> column 0, end 1 -> 9;
+        ix=1: start -1 -> column 1 (a clamp to 0 would include the 9), end 2 -> 1;
+        ix=2: columns [0,3) of the row as the in-place pass has left it: [9,1,5] -> 9."""
+    x = np.array([[1, 2, 3, 4, 5], [10, 9, 8, 7, 6], [11, 12, 13, 14, 15], [20, 19, 18, 17, 16],
+                  [21, 22, 23, 24, 25]], np.uint8).reshape(5, 5, 1)
+    got = oracle.maxpool(x, (3, 3), (2, 2), pads=(1, 1, 1, 1), out_hw=(3, 3))
+    np.testing.assert_array_equal(got[:, :, 0], np.array([[10, 9, 7], [20, 19, 17], [22, 24, 25]], np.uint8))
+    # and against the windowed maximum with the padding excluded, on random data
+    r = rng_for(11)
+    xr = rand_u8(r, (9, 11, 3))
+    got = oracle.maxpool(xr, (3, 3), (2, 2), pads=(1, 1, 1, 1), out_hw=(5, 6))
+    for oy in range(5):
+        for ox in range(6):
+            ys, ye = max(0, 2 * oy - 1), min(2 * oy + 2, 9)
+            xs, xe = max(0, 2 * ox - 1), min(2 * ox + 2, 11)
+            np.testing.assert_array_equal(got[oy, ox], xr[ys:ye, xs:xe].max(axis=(0, 1)))
+    y = np.array([9, 1, 5, 3], np.uint8).reshape(1, 4, 1)
+    got = oracle.maxpool(y, (3, 1), (1, 1), pads=(0, 0, 2, 0), out_hw=(1, 3))
+    np.testing.assert_array_equal(got[0, :, 0], np.array([9, 1, 9], np.uint8))
+
+
 def test_add_matches_exact_integers():
     r = rng_for(10)
     a, b = rand_u8(r, (3, 5, 7, 4)), rand_u8(r, (3, 5, 7, 4))
