@@ -73,6 +73,45 @@ void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bi
                                unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
                                unsigned short stride, signed char flag_relu, signed char flag_batch_norm);
 
+/* ---- calibration of out_shift -------------------------------------------------------
+ * A network that requantises with batch-norm + ReLU chooses, per layer,
+ * out_shift = floor(log2(max |acc * k[c]|)) - 7, the maximum taken over the batch, all
+ * output pixels and all output channels; acc is the layer's accumulator including bias
+ * (what pulp_nn_matmul / pulp_nn_depthwise_generic hand to pulp_nn_bn_quant_u8).  The
+ * reference leaves this to offline tooling; the calls below compute it on the GPU from the
+ * layer's own device tensors, for pulp_nn_hip_set_batch() images.
+ *
+ * result points to two 64-bit words in DEVICE memory, written on the stream:
+ * result[0] = max |acc * k[c]| (64-bit wrapping product, as the 64-bit tree forms it),
+ * result[1] = max(floor(log2(result[0])) - 7, 0), and 0 for a layer whose maximum is 0.
+ * k is an int32_t or int64_t array as the build expects.  The geometry arguments have the
+ * meaning they have in pulp_nn_conv_Ho_parallel (a pointwise layer is a 1x1 kernel with
+ * stride 1 and no padding; a linear layer is a pointwise layer on a 1x1 image) and in
+ * pulp_nn_depthwise_generic.
+ *
+ * workspace: device memory for the partial maxima, 8-byte aligned, at least
+ * pulp_nn_hip_calib_workspace_bytes(batch * dim_out_x * dim_out_y * ch_out) bytes (one
+ * 8-byte slot per 65536 outputs); its previous contents do not matter.  Calls that share a
+ * workspace must not overlap in time. */
+unsigned long long pulp_nn_hip_calib_workspace_bytes(unsigned long long n_outputs);
+
+void pulp_nn_hip_calib_conv(const unsigned char *pInBuffer, const signed char *bias, const signed char *pWeight,
+                            const void *k, unsigned short dim_in_x, unsigned short dim_in_y, unsigned short ch_in,
+                            unsigned short dim_out_x, unsigned short dim_out_y, unsigned short ch_out,
+                            unsigned short dim_kernel_x, unsigned short dim_kernel_y, unsigned short padding_y_top,
+                            unsigned short padding_x_left, unsigned short stride_x, unsigned short stride_y,
+                            void *workspace, unsigned long long workspace_bytes, unsigned long long *result);
+
+/* Depthwise layer (one [ky][kx] filter per channel).  input_is_hwc = 0: CHW input as
+ * pulp_nn_depthwise_generic takes it; 1: HWC input as pulp_nn_hip_depthwise_hwc takes it. */
+void pulp_nn_hip_calib_depthwise(const unsigned char *Im_in, const signed char *bias, const signed char *wt,
+                                 const void *k, unsigned short dim_im_in_x, unsigned short dim_im_in_y,
+                                 unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
+                                 unsigned short dim_kernel_x, unsigned short dim_kernel_y, unsigned short padding_y_top,
+                                 unsigned short padding_x_left, unsigned short stride_x, unsigned short stride_y,
+                                 int input_is_hwc, void *workspace, unsigned long long workspace_bytes,
+                                 unsigned long long *result);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,12 @@ class PulpNN:
         L.pulp_nn_hip_hwc_to_chw.restype = None
         L.pulp_nn_hip_depthwise_hwc.argtypes = [_PTR] * 6 + [_U16] * 8 + [_I8, _I8]
         L.pulp_nn_hip_depthwise_hwc.restype = None
+        _U64 = C.c_uint64
+        L.pulp_nn_hip_calib_workspace_bytes.argtypes, L.pulp_nn_hip_calib_workspace_bytes.restype = [_U64], _U64
+        L.pulp_nn_hip_calib_conv.argtypes = [_PTR] * 4 + [_U16] * 12 + [_PTR, _U64, _PTR]
+        L.pulp_nn_hip_calib_conv.restype = None
+        L.pulp_nn_hip_calib_depthwise.argtypes = [_PTR] * 4 + [_U16] * 11 + [_INT, _PTR, _U64, _PTR]
+        L.pulp_nn_hip_calib_depthwise.restype = None
         assert L.pulp_nn_hip_bn_bits() == bn_bits
 
     # -- added entry points ------------------------------------------------
@@ -136,6 +142,23 @@ class PulpNN:
         PulpNNError (unsupported) for geometries without a fused kernel."""
         self._call("pulp_nn_hip_depthwise_hwc", _ptr(x), _ptr(bias), _ptr(out), _ptr(wt), _ptr(k), _ptr(lam), out_mult,
                    out_shift, dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, stride, flag_relu, flag_batch_norm)
+
+    # -- calibration ---------------------------------------------------------
+    def calib_workspace_bytes(self, n_outputs):
+        return int(self._lib.pulp_nn_hip_calib_workspace_bytes(int(n_outputs)))
+
+    def calib_conv(self, x, bias, w, k, dim_in_x, dim_in_y, ch_in, dim_out_x, dim_out_y, ch_out, kx, ky, pad_top,
+                   pad_left, stride_x, stride_y, workspace, workspace_bytes, result):
+        """result (device, 2 x uint64) <- max |acc * k|, and the out_shift floor(log2(max)) - 7 derived from it."""
+        self._call("pulp_nn_hip_calib_conv", _ptr(x), _ptr(bias), _ptr(w), _ptr(k), dim_in_x, dim_in_y, ch_in,
+                   dim_out_x, dim_out_y, ch_out, kx, ky, pad_top, pad_left, stride_x, stride_y, _ptr(workspace),
+                   int(workspace_bytes), _ptr(result))
+
+    def calib_depthwise(self, x, bias, wt, k, dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, kx, ky, pad_top, pad_left,
+                        stride_x, stride_y, input_is_hwc, workspace, workspace_bytes, result):
+        self._call("pulp_nn_hip_calib_depthwise", _ptr(x), _ptr(bias), _ptr(wt), _ptr(k), dim_in_x, dim_in_y, ch,
+                   dim_out_x, dim_out_y, kx, ky, pad_top, pad_left, stride_x, stride_y, int(input_is_hwc),
+                   _ptr(workspace), int(workspace_bytes), _ptr(result))
 
     # -- the reference API ---------------------------------------------------
     def _conv(self, name, pIn, pIm2Col, bias, pOut, pWeight, k, lam, *scalars):

@@ -16,6 +16,10 @@
 #include "../../include/32bit/pulp_nn_kernels.h"
 #endif
 
+#include <atomic>
+#include <mutex>
+
+#include "calib.h"
 #include "depthwise.h"
 #include "igemm.h"
 #include "linear_skinny.h"
@@ -70,14 +74,18 @@ bool epi_args(int mode, const bn_t *k, const bn_t *lambda, uint16_t out_mult, in
   return e->shift >= 0 && e->shift < lim;
 }
 
+// Compute units of the current device.  Cached per process; concurrent first calls compute the
+// same value, so a relaxed atomic is enough.
 int num_cus()
 {
-  static int n = 0;
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
   if (!n) {
     int dev = 0;
     hipDeviceProp_t p;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) n = p.multiProcessorCount;
     if (n <= 0) n = 256;
+    cached.store(n, std::memory_order_relaxed);
   }
   return n;
 }
@@ -166,10 +174,16 @@ void launch_smallk(int mode, bool rows, ConvGeom &g, const EpiArgs &e, hipStream
 template <auto KERN>
 void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t lds, hipStream_t s)
 {
-  static size_t limit = 65536;
-  if (lds > limit) {
-    (void)hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    limit = lds;
+  // (raising the limit twice from two host threads is harmless; the mutex keeps the cached value
+  // from running ahead of the attribute)
+  static std::mutex mu;
+  static std::atomic<size_t> limit{65536};
+  if (lds > limit.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (lds > limit.load(std::memory_order_relaxed)) {
+      (void)hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      limit.store(lds, std::memory_order_release);
+    }
   }
   hipLaunchKernelGGL(KERN, grid, block, lds, s, g, e);
 }
@@ -584,6 +598,54 @@ bool pool_geom(const char *fn, PoolGeom *g, uint8_t *in, uint8_t *out, uint16_t 
   return true;
 }
 
+// ---- calibration ---------------------------------------------------------------------
+
+// Shared body of the calibration entry points.  partial: device memory for `slots_avail` partial maxima.
+void calib_common(const char *fn, CalibGeom &g, unsigned long long *partial, unsigned long long slots_avail,
+                  unsigned long long *result)
+{
+  if (!g.in || !g.w || !g.k || !result) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "null pointer");
+  if (g.W <= 0 || g.H <= 0 || g.Ci <= 0 || g.Wo <= 0 || g.Ho <= 0 || g.Co <= 0 || g.kx <= 0 || g.ky <= 0 || g.sx <= 0 ||
+      g.sy <= 0)
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
+  g.total = (long long)g_batch * g.Ho * g.Wo * g.Co;
+  g.in_img = (long long)g.H * g.W * g.Ci;
+  const unsigned long long slots = ((unsigned long long)g.total + CALIB_CHUNK - 1) / CALIB_CHUNK;
+  if (slots > 0x7fffffffull) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+  if (!partial || slots > slots_avail)
+    return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn,
+                     "layer too large for the partial-maximum buffer (one 8-byte slot per 65536 outputs)");
+  hipLaunchKernelGGL(calib_absmax_kernel, dim3((unsigned)slots), dim3(256), 0, g_stream, g, partial);
+  hipLaunchKernelGGL(calib_final_kernel, dim3(1), dim3(256), 0, g_stream, partial, (int)slots, result);
+  check_launch(fn);
+}
+
+CalibGeom calib_conv_geom(const unsigned char *in, const signed char *bias, const signed char *w, const void *k,
+                          unsigned short dim_in_x, unsigned short dim_in_y, unsigned short ch_in,
+                          unsigned short dim_out_x, unsigned short dim_out_y, unsigned short ch_out,
+                          unsigned short kx, unsigned short ky, unsigned short pt, unsigned short pl,
+                          unsigned short sx, unsigned short sy)
+{
+  CalibGeom g = {};
+  g.in = in;
+  g.w = (const int8_t *)w;
+  g.bias = (const int8_t *)bias;
+  g.k = (const bn_t *)k;
+  g.H = dim_in_y;
+  g.W = dim_in_x;
+  g.Ci = ch_in;
+  g.Ho = dim_out_y;
+  g.Wo = dim_out_x;
+  g.Co = ch_out;
+  g.kx = kx;
+  g.ky = ky;
+  g.pt = pt;
+  g.pl = pl;
+  g.sx = sx;
+  g.sy = sy;
+  return g;
+}
+
 }  // namespace
 
 // ---- added entry points -----------------------------------------------------------
@@ -644,6 +706,40 @@ void pulp_nn_hip_hwc_to_chw(const unsigned char *in_hwc, unsigned char *out_chw,
   hipLaunchKernelGGL(hwc_to_chw_kernel, dim3((unsigned)total), dim3(256), 0, g_stream, in_hwc, out_chw, (int)dim_y,
                      (int)dim_x, (int)ch, (int)pad_top, (int)pad_bottom, tiles_p, tiles_c);
   check_launch(__func__);
+}
+
+unsigned long long pulp_nn_hip_calib_workspace_bytes(unsigned long long n_outputs)
+{
+  return ((n_outputs + CALIB_CHUNK - 1) / CALIB_CHUNK) * sizeof(unsigned long long);
+}
+
+void pulp_nn_hip_calib_conv(const unsigned char *pInBuffer, const signed char *bias, const signed char *pWeight,
+                            const void *k, unsigned short dim_in_x, unsigned short dim_in_y, unsigned short ch_in,
+                            unsigned short dim_out_x, unsigned short dim_out_y, unsigned short ch_out,
+                            unsigned short dim_kernel_x, unsigned short dim_kernel_y, unsigned short padding_y_top,
+                            unsigned short padding_x_left, unsigned short stride_x, unsigned short stride_y,
+                            void *workspace, unsigned long long workspace_bytes, unsigned long long *result)
+{
+  CalibGeom g = calib_conv_geom(pInBuffer, bias, pWeight, k, dim_in_x, dim_in_y, ch_in, dim_out_x, dim_out_y, ch_out,
+                                dim_kernel_x, dim_kernel_y, padding_y_top, padding_x_left, stride_x, stride_y);
+  REQUIRE(aligned(workspace, 8) && aligned(result, 8), PULP_NN_HIP_ERR_ARGUMENT, "workspace and result must be 8-byte aligned");
+  calib_common(__func__, g, (unsigned long long *)workspace, workspace_bytes / sizeof(unsigned long long), result);
+}
+
+void pulp_nn_hip_calib_depthwise(const unsigned char *Im_in, const signed char *bias, const signed char *wt,
+                                 const void *k, unsigned short dim_im_in_x, unsigned short dim_im_in_y,
+                                 unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
+                                 unsigned short dim_kernel_x, unsigned short dim_kernel_y, unsigned short padding_y_top,
+                                 unsigned short padding_x_left, unsigned short stride_x, unsigned short stride_y,
+                                 int input_is_hwc, void *workspace, unsigned long long workspace_bytes,
+                                 unsigned long long *result)
+{
+  CalibGeom g = calib_conv_geom(Im_in, bias, wt, k, dim_im_in_x, dim_im_in_y, ch, dim_im_out_x, dim_im_out_y, ch,
+                                dim_kernel_x, dim_kernel_y, padding_y_top, padding_x_left, stride_x, stride_y);
+  g.depthwise = 1;
+  g.chw_in = !input_is_hwc;
+  REQUIRE(aligned(workspace, 8) && aligned(result, 8), PULP_NN_HIP_ERR_ARGUMENT, "workspace and result must be 8-byte aligned");
+  calib_common(__func__, g, (unsigned long long *)workspace, workspace_bytes / sizeof(unsigned long long), result);
 }
 
 // ---- the reference API ------------------------------------------------------------

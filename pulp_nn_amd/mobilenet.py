@@ -19,7 +19,7 @@ import os
 
 import numpy as np
 
-from .api import PulpNNError
+from . import network
 
 WIDTHS = (32, 64, 64, 128, 128, 256, 256, 256, 256, 256, 256, 512, 512)
 STRIDE2_BLOCKS = (2, 4, 6, 12)   # 1-based
@@ -77,58 +77,39 @@ def build(batch=256, shifts=None):
     return net
 
 
-class Runner:
-    """Uploads the parameters once and runs the chain on the GPU through the C API."""
+def descriptor(net):
+    """The chain as a layer table for network.Runner (see network.py for the format)."""
+    layers, prev = [], "input"
+    for L in net["layers"]:
+        s = L["stride"]
+        common = dict(name=L["name"], w=L["w"], bias=L["bias"], k=L["k"], lam=L["lam"], relu=1, bn=1, mult=0,
+                      shift=L["shift"])
+        common["in"] = prev
+        if L["kind"] == "conv":
+            layers.append(dict(op="conv", pads=(1, 1, 1, 1), strides=(s, s), out_hw=(L["hout"], L["hout"]), **common))
+        elif L["kind"] == "dw":
+            layers.append(dict(op="depthwise", pads=(1, 1, 1, 1), strides=(s, s), out_hw=(L["hout"], L["hout"]), **common))
+        else:
+            layers.append(dict(op="pointwise", **common))
+        prev = L["name"]
+    layers.append({"op": "avgpool", "name": "pool", "in": prev, "kernel": (4, 4), "strides": (4, 4), "out_hw": (1, 1)})
+    layers.append({"op": "linear_out_32", "name": "fc", "in": "pool", "w": net["fc_w"], "bias32": net["fc_bias"]})
+    return layers
+
+
+class Runner(network.Runner):
+    """The configuration-3 chain on the generic runner.  fused: depthwise layers read the HWC
+    output of the previous layer directly (pulp_nn_hip_depthwise_hwc) where the library has a
+    kernel for it; otherwise, and with fused=False, the chain is the reference's:
+    pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic."""
 
     def __init__(self, nn, net, fused=True):
-        import torch
-        self.nn, self.net, self.torch = nn, net, torch
-        # fused: depthwise layers read the HWC output of the previous layer directly
-        # (pulp_nn_hip_depthwise_hwc) where the library has a kernel for it; otherwise, and with
-        # fused=False, the chain is the reference's: pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic
-        self.fused, self.unfused = fused, set()
-        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-        self.params = [dict(w=dev(L["w"]), bias=dev(L["bias"]), k=dev(L["k"]), lam=dev(L["lam"]))
-                       for L in net["layers"]]
-        self.fc_w, self.fc_bias = dev(net["fc_w"]), dev(net["fc_bias"])
-        B = net["batch"]
-        u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device="cuda")
-        self.act = [u8(B, L["hout"], L["hout"], L["cout"]) for L in net["layers"]]
-        self.chw = {i: u8(B, L["cin"], L["hin"], L["hin"]) for i, L in enumerate(net["layers"]) if L["kind"] == "dw"}
-        self.pooled = u8(B, 512)
-        self.logits = torch.empty((B, 1000), dtype=torch.int32, device="cuda")
+        self.net = net
+        super().__init__(nn, descriptor(net), (128, 128, 3), net["batch"], fused=fused)
+        self.logits = self.act["fc"].view(net["batch"], 1000)
+        self.activations = [self.act[L["name"]] for L in net["layers"]]
 
     def run(self, x):
         """x: device tensor B,128,128,3 uint8.  Returns the int32 logits tensor (B,1000)."""
-        nn, B = self.nn, self.net["batch"]
-        nn.set_batch(B)
-        cur = x
-        for i, (L, P) in enumerate(zip(self.net["layers"], self.params)):
-            out = self.act[i]
-            hi, ho, ci, co, s = L["hin"], L["hout"], L["cin"], L["cout"], L["stride"]
-            if L["kind"] == "conv":
-                nn.pulp_nn_conv_Ho_parallel(cur, None, P["bias"], out, P["w"], P["k"], P["lam"], 0, L["shift"],
-                                            hi, hi, ci, ho, ho, co, 3, 3, 1, 1, 1, 1, s, s, 1, 1)
-            elif L["kind"] == "dw":
-                if self.fused and i not in self.unfused:
-                    try:
-                        # layout change fused into the depthwise kernel
-                        nn.depthwise_hwc(cur, P["bias"], out, P["w"], P["k"], P["lam"], 0, L["shift"],
-                                         hi, hi, ci, ho, ho, s, 1, 1)
-                        cur = out
-                        continue
-                    except PulpNNError as err:
-                        if err.code != 2:
-                            raise
-                        self.unfused.add(i)   # no fused kernel for this geometry
-                chw = self.chw[i]
-                nn.hwc_to_chw(cur, chw, hi, hi, ci)
-                nn.pulp_nn_depthwise_generic(chw, None, P["bias"], out, P["w"], None, P["k"], P["lam"], 0, L["shift"],
-                                             hi, hi, ci, ho, ho, co, 3, 3, 1, 1, 1, 1, s, s, 1, 1)
-            else:
-                nn.pulp_nn_pointwise_HoWo_parallel(cur, None, P["bias"], out, P["w"], P["k"], P["lam"], 0, L["shift"],
-                                                   hi, hi, ci, ho, ho, co, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1)
-            cur = out
-        nn.pulp_nn_avgpool(cur, self.pooled, 0, 0, 0, 4, 4, 512, 1, 1, 4, 4, 0, 0, 0, 0, 4, 4, 0)
-        nn.pulp_nn_linear_out_32(self.pooled, self.fc_bias, self.logits, self.fc_w, 512, 1000)
+        super().run(x)
         return self.logits

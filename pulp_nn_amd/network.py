@@ -1,0 +1,236 @@
+"""A small layer-table format for chained int8 networks and a runner that executes it on the
+GPU through the C API (what generated deployment code does by hand with the reference:
+one pulp_nn_* call per layer on caller-owned buffers).
+
+A network is a list of layer dicts.  Every layer has "op", "name" and "in" (the name of the
+tensor it reads; the network input is called "input"; "add" takes a pair of names) and
+produces the tensor called like the layer.  Activations are HWC uint8, batch outermost.
+
+  op            parameters
+  conv          w [Co,ky,kx,Ci] int8, bias [Co] int8 or None, pads (t,b,l,r), strides (sx,sy),
+                requantisation (below)                      -> pulp_nn_conv_Ho_parallel
+  pointwise     w [Co,1,1,Ci], bias, requantisation        -> pulp_nn_pointwise_HoWo_parallel
+  depthwise     w [C,ky,kx], bias, pads, strides, requantisation.  The tensor it reads is HWC
+                like all others; the runner changes the layout (pulp_nn_hip_hwc_to_chw +
+                pulp_nn_depthwise_generic) or, for 3x3 / padding 1 layers the library has a
+                fused kernel for, calls pulp_nn_hip_depthwise_hwc
+  maxpool       kernel (kx,ky), strides, pads, out_hw      -> pulp_nn_maxpool
+  avgpool       kernel, strides, pads, out_hw, lam, shift, add, requant -> pulp_nn_avgpool
+  add           in = (a, b), m1, m2, shift                 -> pulp_nn_add
+  linear        w [N,K] int8, bias, requantisation; reads its input flattened per image
+                                                           -> pulp_nn_linear
+  linear_out_32 w [N,K], bias32 [N] int32 or None; int32 output -> pulp_nn_linear_out_32
+
+Requantisation keys: relu, bn (the two flags), k, lam ([Co] arrays for bn), mult (out_mult),
+shift (out_shift).  shift = None on a bn layer means "to be calibrated": Runner.calibrate()
+sets it to floor(log2(max |acc * k|)) - 7 over the batch it is given, computed on the GPU
+(pulp_nn_hip_calib_conv / pulp_nn_hip_calib_depthwise), layer by layer along the chain.
+"""
+import numpy as np
+
+from .api import PulpNNError
+
+CONV_LIKE = ("conv", "pointwise", "depthwise", "linear")
+
+
+def out_size(n, k, s, p0, p1):
+    return (n + p0 + p1 - k) // s + 1
+
+
+def infer_shapes(layers, input_shape):
+    """{tensor name: (H, W, C)} for the input and every layer output (linear outputs are (1, 1, N))."""
+    shapes = {"input": tuple(input_shape)}
+    for L in layers:
+        op = L["op"]
+        src = L["in"][0] if op == "add" else L["in"]
+        H, W, Cc = shapes[src]
+        if op in ("conv", "pointwise"):
+            Co, ky, kx, Ci = L["w"].shape
+            assert Ci == Cc, (L["name"], Ci, Cc)
+            if op == "pointwise":
+                shapes[L["name"]] = (H, W, Co)
+            else:
+                pt, pb, pl, pr = L["pads"]
+                sx, sy = L["strides"]
+                shapes[L["name"]] = L.get("out_hw", (out_size(H, ky, sy, pt, pb), out_size(W, kx, sx, pl, pr))) + (Co,)
+        elif op == "depthwise":
+            Cw, ky, kx = L["w"].shape
+            assert Cw == Cc, (L["name"], Cw, Cc)
+            pt, pb, pl, pr = L["pads"]
+            sx, sy = L["strides"]
+            shapes[L["name"]] = L.get("out_hw", (out_size(H, ky, sy, pt, pb), out_size(W, kx, sx, pl, pr))) + (Cc,)
+        elif op in ("maxpool", "avgpool"):
+            shapes[L["name"]] = tuple(L["out_hw"]) + (Cc,)
+        elif op == "add":
+            assert shapes[L["in"][1]] == (H, W, Cc), L["name"]
+            shapes[L["name"]] = (H, W, Cc)
+        elif op in ("linear", "linear_out_32"):
+            N, K = L["w"].shape
+            assert K == H * W * Cc, (L["name"], K, H * W * Cc)
+            shapes[L["name"]] = (1, 1, N)
+        else:
+            raise ValueError("unknown op %r" % op)
+    return shapes
+
+
+class Runner:
+    """Uploads the parameters once, owns the activation buffers and queues the chain."""
+
+    def __init__(self, nn, layers, input_shape, batch, fused=True):
+        import torch
+        self.nn, self.layers, self.batch, self.torch = nn, layers, batch, torch
+        self.fused, self.unfused = fused, set()
+        self.shapes = infer_shapes(layers, input_shape)
+        bn_np = np.int64 if nn.bn_bits == 64 else np.int32
+
+        def dev(a, dtype=None):
+            return None if a is None else torch.from_numpy(np.ascontiguousarray(a, dtype=dtype)).cuda()
+
+        self.params = []
+        for L in layers:
+            P = {}
+            if "w" in L:
+                P["w"] = dev(L["w"], np.int8)
+            if L["op"] == "linear_out_32":
+                P["bias"] = dev(L.get("bias32"), np.int32)
+            elif "bias" in L:
+                P["bias"] = dev(L["bias"], np.int8)
+            if L.get("k") is not None:
+                P["k"], P["lam"] = dev(L["k"], bn_np), dev(L["lam"], bn_np)
+            self.params.append(P)
+        self.act = {}
+        for L in layers:
+            H, W, Cc = self.shapes[L["name"]]
+            dt = torch.int32 if L["op"] == "linear_out_32" else torch.uint8
+            self.act[L["name"]] = torch.empty((batch, H, W, Cc), dtype=dt, device="cuda")
+        self.chw = {}
+        for L in layers:
+            if L["op"] == "depthwise":
+                H, W, Cc = self.shapes[L["in"]]
+                self.chw[L["name"]] = torch.empty((batch, Cc, H, W), dtype=torch.uint8, device="cuda")
+        self._calib = None
+
+    # -- one layer ------------------------------------------------------------------------
+    def _requant_args(self, L, P):
+        relu, bn = L.get("relu", 0), L.get("bn", 0)
+        if relu and bn and L.get("shift") is None:
+            raise ValueError("layer %s has no out_shift: run calibrate() first" % L["name"])
+        return P.get("k"), P.get("lam"), L.get("mult", 0), L.get("shift", 0) or 0, relu, bn
+
+    def _queue(self, i, tensors):
+        L, P, nn = self.layers[i], self.params[i], self.nn
+        op, out = L["op"], self.act[L["name"]]
+        if op == "add":
+            a, b = tensors[L["in"][0]], tensors[L["in"][1]]
+            H, W, Cc = self.shapes[L["name"]]
+            nn.pulp_nn_add(a, b, out, L["m1"], L["m2"], L["shift"], H, W, Cc)
+            return out
+        cur = tensors[L["in"]]
+        H, W, Cc = self.shapes[L["in"]]
+        Ho, Wo, Co = self.shapes[L["name"]]
+        if op in ("conv", "pointwise"):
+            k, lam, mult, shift, relu, bn = self._requant_args(L, P)
+            if op == "conv":
+                ky, kx = L["w"].shape[1:3]
+                pt, pb, pl, pr = L["pads"]
+                sx, sy = L["strides"]
+                nn.pulp_nn_conv_Ho_parallel(cur, None, P.get("bias"), out, P["w"], k, lam, mult, shift, W, H, Cc, Wo, Ho,
+                                            Co, kx, ky, pt, pb, pl, pr, sx, sy, relu, bn)
+            else:
+                nn.pulp_nn_pointwise_HoWo_parallel(cur, None, P.get("bias"), out, P["w"], k, lam, mult, shift, W, H, Cc,
+                                                   Wo, Ho, Co, 1, 1, 0, 0, 0, 0, 1, 1, relu, bn)
+        elif op == "depthwise":
+            k, lam, mult, shift, relu, bn = self._requant_args(L, P)
+            ky, kx = L["w"].shape[1:3]
+            pt, pb, pl, pr = L["pads"]
+            sx, sy = L["strides"]
+            fusable = (ky, kx) == (3, 3) and tuple(L["pads"]) == (1, 1, 1, 1) and sx == sy
+            if self.fused and fusable and i not in self.unfused:
+                try:
+                    nn.depthwise_hwc(cur, P.get("bias"), out, P["w"], k, lam, mult, shift, W, H, Cc, Wo, Ho, sx, relu, bn)
+                    return out
+                except PulpNNError as err:
+                    if err.code != 2:
+                        raise
+                    self.unfused.add(i)    # no fused kernel for this geometry
+            chw = self.chw[L["name"]]
+            nn.hwc_to_chw(cur, chw, W, H, Cc)
+            nn.pulp_nn_depthwise_generic(chw, None, P.get("bias"), out, P["w"], None, k, lam, mult, shift, W, H, Cc,
+                                         Wo, Ho, Cc, kx, ky, pt, pb, pl, pr, sx, sy, relu, bn)
+        elif op == "maxpool":
+            kx, ky = L["kernel"]
+            sx, sy = L["strides"]
+            pt, pb, pl, pr = L.get("pads", (0, 0, 0, 0))
+            nn.pulp_nn_maxpool(cur, out, W, H, Cc, Wo, Ho, kx, ky, pt, pb, pl, pr, sx, sy)
+        elif op == "avgpool":
+            kx, ky = L["kernel"]
+            sx, sy = L["strides"]
+            pt, pb, pl, pr = L.get("pads", (0, 0, 0, 0))
+            nn.pulp_nn_avgpool(cur, out, L.get("lam", 0), L.get("shift", 0), L.get("add", 0), W, H, Cc, Wo, Ho, kx, ky,
+                               pt, pb, pl, pr, sx, sy, L.get("requant", 0))
+        elif op == "linear":
+            k, lam, mult, shift, relu, bn = self._requant_args(L, P)
+            nn.pulp_nn_linear(cur, P.get("bias"), out, P["w"], k, lam, mult, shift, H * W * Cc, Co, relu, bn)
+        elif op == "linear_out_32":
+            nn.pulp_nn_linear_out_32(cur, P.get("bias"), out, P["w"], H * W * Cc, Co)
+        else:
+            raise ValueError(op)
+        return out
+
+    def run(self, x):
+        """x: device tensor batch,H,W,C uint8.  Queues every layer; returns the last layer's tensor."""
+        self.nn.set_batch(self.batch)
+        tensors = {"input": x}
+        out = x
+        for i, L in enumerate(self.layers):
+            out = tensors[L["name"]] = self._queue(i, tensors)
+        return out
+
+    # -- calibration ------------------------------------------------------------------------
+    def _calib_buffers(self):
+        if self._calib is None:
+            torch = self.torch
+            most = max(self.batch * int(np.prod(self.shapes[L["name"]])) for L in self.layers)
+            nbytes = self.nn.calib_workspace_bytes(most)
+            self._calib = (torch.empty(nbytes // 8 + 1, dtype=torch.int64, device="cuda"), nbytes,
+                           torch.zeros(2, dtype=torch.int64, device="cuda"))
+        return self._calib
+
+    def layer_absmax(self, i, tensors):
+        """(max |acc * k|, derived out_shift) of conv-like layer i on the GPU."""
+        L, P, nn = self.layers[i], self.params[i], self.nn
+        ws, nbytes, res = self._calib_buffers()
+        cur = tensors[L["in"]]
+        H, W, Cc = self.shapes[L["in"]]
+        Ho, Wo, Co = self.shapes[L["name"]]
+        nn.set_batch(self.batch)
+        if L["op"] == "depthwise":
+            ky, kx = L["w"].shape[1:3]
+            pt, _, pl, _ = L["pads"]
+            sx, sy = L["strides"]
+            nn.calib_depthwise(cur, P.get("bias"), P["w"], P["k"], W, H, Cc, Wo, Ho, kx, ky, pt, pl, sx, sy, 1, ws,
+                               nbytes, res)
+        elif L["op"] == "linear":
+            nn.calib_conv(cur, P.get("bias"), P["w"], P["k"], 1, 1, H * W * Cc, 1, 1, Co, 1, 1, 0, 0, 1, 1, ws, nbytes, res)
+        else:
+            ky, kx = L["w"].shape[1:3]
+            pt, _, pl, _ = L.get("pads", (0, 0, 0, 0))
+            sx, sy = L.get("strides", (1, 1))
+            nn.calib_conv(cur, P.get("bias"), P["w"], P["k"], W, H, Cc, Wo, Ho, Co, kx, ky, pt, pl, sx, sy, ws, nbytes, res)
+        nn.sync()
+        m, shift = (int(v) for v in res.cpu().numpy().view(np.uint64))
+        return m, shift
+
+    def calibrate(self, x, force=False):
+        """Runs the chain on x and gives every batch-norm layer without an out_shift (all of them with
+        force=True) the shift floor(log2(max |acc * k|)) - 7 measured on this batch.  Returns {name: shift}."""
+        self.nn.set_batch(self.batch)
+        tensors = {"input": x}
+        chosen = {}
+        for i, L in enumerate(self.layers):
+            if L["op"] in CONV_LIKE and L.get("relu") and L.get("bn") and (force or L.get("shift") is None):
+                _, L["shift"] = self.layer_absmax(i, tensors)
+                chosen[L["name"]] = L["shift"]
+            tensors[L["name"]] = self._queue(i, tensors)
+        self.nn.sync()
+        return chosen

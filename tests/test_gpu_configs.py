@@ -83,7 +83,7 @@ def test_config3_mobilenet_batch256():
     # two images through the oracle chain, every intermediate layer compared
     want_logits, want_layers = cfg3_oracle.forward(net, net["x"][:2], keep=True)
     for i, (Ld, w) in enumerate(zip(net["layers"], want_layers)):
-        assert_same(runner.act[i][:2].cpu().numpy(), w, "config 3 layer %s" % Ld["name"])
+        assert_same(runner.activations[i][:2].cpu().numpy(), w, "config 3 layer %s" % Ld["name"])
     assert_same(got[:2], want_logits, "config 3 logits")
     check_digest("cfg3_b256_logits", got)
     assert not runner.unfused, "depthwise layers without a fused kernel: %s" % sorted(runner.unfused)
@@ -115,7 +115,7 @@ def test_config3_chain_in_a_hip_graph():
     try:
         for i in range(3):
             runner.logits.fill_(-1)
-            for a in runner.act:
+            for a in runner.activations:
                 a.random_(0, 255)      # eager work between the replays; every activation is rewritten by the graph
             torch.cuda.synchronize()
             graph.replay()
