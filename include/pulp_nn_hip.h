@@ -112,6 +112,23 @@ void pulp_nn_hip_calib_depthwise(const unsigned char *Im_in, const signed char *
                                  int input_is_hwc, void *workspace, unsigned long long workspace_bytes,
                                  unsigned long long *result);
 
+/* pulp_nn_hip_calib_conv for callers that cannot allocate device memory or carry a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): no counterpart in the reference.  Same arguments and same result as
+ * pulp_nn_hip_calib_conv without the workspace: the partial maxima go to a fixed array of
+ * 8192 slots (64 KiB) that the library holds in the device memory of every GPU it runs on
+ * until the process ends.  The call allocates and frees nothing.  A layer with more than
+ * 8192 * 65536 outputs (batch * dim_out_x * dim_out_y * ch_out) is rejected with
+ * PULP_NN_HIP_ERR_ARGUMENT.  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (different streams or host threads) race and must be serialised by the
+ * caller. */
+void pulp_nn_hip_calib_conv_static(const unsigned char *pInBuffer, const signed char *bias, const signed char *pWeight,
+                                   const void *k, unsigned short dim_in_x, unsigned short dim_in_y,
+                                   unsigned short ch_in, unsigned short dim_out_x, unsigned short dim_out_y,
+                                   unsigned short ch_out, unsigned short dim_kernel_x, unsigned short dim_kernel_y,
+                                   unsigned short padding_y_top, unsigned short padding_x_left,
+                                   unsigned short stride_x, unsigned short stride_y, unsigned long long *result);
+
 #ifdef __cplusplus
 }
 #endif

@@ -90,6 +90,8 @@ class PulpNN:
         L.pulp_nn_hip_calib_conv.restype = None
         L.pulp_nn_hip_calib_depthwise.argtypes = [_PTR] * 4 + [_U16] * 11 + [_INT, _PTR, _U64, _PTR]
         L.pulp_nn_hip_calib_depthwise.restype = None
+        L.pulp_nn_hip_calib_conv_static.argtypes = [_PTR] * 4 + [_U16] * 12 + [_PTR]
+        L.pulp_nn_hip_calib_conv_static.restype = None
         assert L.pulp_nn_hip_bn_bits() == bn_bits
 
     # -- added entry points ------------------------------------------------
@@ -159,6 +161,12 @@ class PulpNN:
         self._call("pulp_nn_hip_calib_depthwise", _ptr(x), _ptr(bias), _ptr(wt), _ptr(k), dim_in_x, dim_in_y, ch,
                    dim_out_x, dim_out_y, kx, ky, pad_top, pad_left, stride_x, stride_y, int(input_is_hwc),
                    _ptr(workspace), int(workspace_bytes), _ptr(result))
+
+    def calib_conv_static(self, x, bias, w, k, dim_in_x, dim_in_y, ch_in, dim_out_x, dim_out_y, ch_out, kx, ky,
+                          pad_top, pad_left, stride_x, stride_y, result):
+        """calib_conv without a workspace argument: the library's fixed scratch array holds the partial maxima."""
+        self._call("pulp_nn_hip_calib_conv_static", _ptr(x), _ptr(bias), _ptr(w), _ptr(k), dim_in_x, dim_in_y, ch_in,
+                   dim_out_x, dim_out_y, ch_out, kx, ky, pad_top, pad_left, stride_x, stride_y, _ptr(result))
 
     # -- the reference API ---------------------------------------------------
     def _conv(self, name, pIn, pIm2Col, bias, pOut, pWeight, k, lam, *scalars):

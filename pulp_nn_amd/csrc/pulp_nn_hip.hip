@@ -600,6 +600,35 @@ bool pool_geom(const char *fn, PoolGeom *g, uint8_t *in, uint8_t *out, uint16_t 
 
 // ---- calibration ---------------------------------------------------------------------
 
+// Device memory of the allocation-free calibration entry point: one partial maximum per
+// workgroup.  In host code the array's name only stands for the symbol; its device address
+// comes from hipGetSymbolAddress, once per device (every GPU holds its own copy).
+#define CALIB_STATIC_SLOTS 8192
+static __device__ __align__(256) unsigned long long scratch[CALIB_STATIC_SLOTS];
+
+unsigned long long *static_scratch(const char *fn)
+{
+  constexpr int MAX_DEV = 64;
+  static std::mutex mu;
+  static unsigned long long *ptr[MAX_DEV] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+    set_error(PULP_NN_HIP_ERR_RUNTIME, fn, "cannot identify the current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error(PULP_NN_HIP_ERR_RUNTIME, fn, hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr[dev] = (unsigned long long *)p;
+  }
+  return ptr[dev];
+}
+
 // Shared body of the calibration entry points.  partial: device memory for `slots_avail` partial maxima.
 void calib_common(const char *fn, CalibGeom &g, unsigned long long *partial, unsigned long long slots_avail,
                   unsigned long long *result)
@@ -724,6 +753,21 @@ void pulp_nn_hip_calib_conv(const unsigned char *pInBuffer, const signed char *b
                                 dim_kernel_x, dim_kernel_y, padding_y_top, padding_x_left, stride_x, stride_y);
   REQUIRE(aligned(workspace, 8) && aligned(result, 8), PULP_NN_HIP_ERR_ARGUMENT, "workspace and result must be 8-byte aligned");
   calib_common(__func__, g, (unsigned long long *)workspace, workspace_bytes / sizeof(unsigned long long), result);
+}
+
+void pulp_nn_hip_calib_conv_static(const unsigned char *pInBuffer, const signed char *bias, const signed char *pWeight,
+                                   const void *k, unsigned short dim_in_x, unsigned short dim_in_y,
+                                   unsigned short ch_in, unsigned short dim_out_x, unsigned short dim_out_y,
+                                   unsigned short ch_out, unsigned short dim_kernel_x, unsigned short dim_kernel_y,
+                                   unsigned short padding_y_top, unsigned short padding_x_left,
+                                   unsigned short stride_x, unsigned short stride_y, unsigned long long *result)
+{
+  CalibGeom g = calib_conv_geom(pInBuffer, bias, pWeight, k, dim_in_x, dim_in_y, ch_in, dim_out_x, dim_out_y, ch_out,
+                                dim_kernel_x, dim_kernel_y, padding_y_top, padding_x_left, stride_x, stride_y);
+  REQUIRE(aligned(result, 8), PULP_NN_HIP_ERR_ARGUMENT, "result must be 8-byte aligned");
+  unsigned long long *partial = static_scratch(__func__);
+  if (!partial) return;
+  calib_common(__func__, g, partial, CALIB_STATIC_SLOTS, result);
 }
 
 void pulp_nn_hip_calib_depthwise(const unsigned char *Im_in, const signed char *bias, const signed char *wt,
