@@ -76,6 +76,79 @@ __device__ __forceinline__ int lds_off(int row, int chunk)
   return row * IGEMM_BK + ((chunk ^ ((row >> 1) & 3)) << 4);
 }
 
+// Epilogue shared by the tiled kernels.  acc[t][s][r] = channel cb + 4*t + r of pixel
+// m0 + wm0 + 16*s + l16, where cb = wn0 + (lane/16)*4*TN; wm0 / wn0: offset of the wave's tile inside
+// the workgroup tile.  wsum is indexed by LDS weight row, cbias / ck_ / cl_ by channel inside the tile.
+// Channel constants are fetched four channels (one MFMA tile row group) at a time to
+// keep the register footprint of the epilogue below that of the main loop.
+template <int TN, int TM, int MODE>
+__device__ __forceinline__ void igemm_epilogue(v4i (&acc)[TN][TM], const ConvGeom &g, const EpiArgs &e, int m0, int n0,
+                                               int wm0, int wn0, int lane, const int *wsum, const int *cbias,
+                                               const bn_t *ck_, const bn_t *cl_)
+{
+  const int l16 = lane & 15, lgrp = lane >> 4;
+  const int cb = wn0 + lgrp * (4 * TN);
+  const bool acc24 = g.K <= 256;  // |acc| <= K * 255 * 128 + 128 < 2^23
+  constexpr int QM = MODE == EPI_OUT32 ? EPI_RAW : MODE;
+  unsigned packed[TM][TN];
+#pragma unroll
+  for (int t = 0; t < TN; t++) {
+    int corr[4];
+    bn_t kk[4], ll[4];
+    bool ks = true;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int c = cb + 4 * t + r;  // channel inside the tile (constants of channels past N are zero)
+      kk[r] = (MODE == EPI_BN) ? ck_[c] : (bn_t)0;
+      ll[r] = (MODE == EPI_BN) ? cl_[c] : (bn_t)0;
+      ks = ks && bn_k_small(kk[r]);
+      corr[r] = cbias[c] + 128 * wsum[wn0 + 16 * t + 4 * lgrp + r];
+    }
+    const bool k_small = __all(ks);  // wave-uniform precondition of the fast batch-norm form
+#pragma unroll
+    for (int s = 0; s < TM; s++) {
+      const int a0 = acc[t][s][0] + corr[0], a1 = acc[t][s][1] + corr[1];
+      const int a2 = acc[t][s][2] + corr[2], a3 = acc[t][s][3] + corr[3];
+      if constexpr (MODE == EPI_OUT32) {
+        const int m = m0 + wm0 + 16 * s + l16;
+        if (m < g.M) {
+          int *o = (int *)g.out + (long long)m * g.N + n0 + cb + 4 * t;
+          const int v[4] = {a0, a1, a2, a3};
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (n0 + cb + 4 * t + r < g.N) o[r] = v[r];
+        }
+      } else {
+        packed[s][t] = acc24 ? requant4<QM, true>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift)
+                             : requant4<QM, false>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift);
+      }
+    }
+  }
+  if constexpr (MODE != EPI_OUT32) {
+    // one copy of the store code per cache policy
+    auto put = [&](auto nt) {
+      constexpr bool NT = decltype(nt)::value;
+#pragma unroll
+      for (int s = 0; s < TM; s++) {
+        const int m = m0 + wm0 + 16 * s + l16;
+        if (m >= g.M) continue;
+        uint8_t *o = (uint8_t *)g.out + (long long)m * g.N + n0 + cb;
+        if (g.vec_store && n0 + cb + 4 * TN <= g.N) {
+          if constexpr (TN == 4) store16<NT>(o, (v4i){(int)packed[s][0], (int)packed[s][1 % TN], (int)packed[s][2 % TN], (int)packed[s][3 % TN]});
+          else if constexpr (TN == 2) store8<NT>(o, (v2i){(int)packed[s][0], (int)packed[s][1 % TN]});
+          else store4<NT>(o, (int)packed[s][0]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4 * TN; c++)
+            if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[s][c >> 2] >> (8 * (c & 3)));
+        }
+      }
+    };
+    if (g.nt) put(std::true_type{});
+    else put(std::false_type{});
+  }
+}
+
 template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N,
                             (WAVES_M * WAVES_N > 8 || TM > 4) ? 1 : (WAVES_M * WAVES_N > 4 || GATHER == GATHER_BYTES ? 2 : IGEMM_MINB))
@@ -373,67 +446,5 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   __syncthreads();
 
   // ---- epilogue ------------------------------------------------------------
-  // acc[t][s][r] = channel cb + 4*t + r of pixel m0 + wave_m*WM + 16*s + l16.
-  // Channel constants are fetched four channels (one MFMA tile row group) at a time to
-  // keep the register footprint of the epilogue below that of the main loop.
-  const int cb = wave_n * WN + lgrp * (4 * TN);
-  const bool acc24 = g.K <= 256;  // |acc| <= K * 255 * 128 + 128 < 2^23
-  constexpr int QM = MODE == EPI_OUT32 ? EPI_RAW : MODE;
-  unsigned packed[TM][TN];
-#pragma unroll
-  for (int t = 0; t < TN; t++) {
-    int corr[4];
-    bn_t kk[4], ll[4];
-    bool ks = true;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int c = cb + 4 * t + r;  // channel inside the tile (constants of channels past N are zero)
-      kk[r] = (MODE == EPI_BN) ? ck_[c] : (bn_t)0;
-      ll[r] = (MODE == EPI_BN) ? cl_[c] : (bn_t)0;
-      ks = ks && bn_k_small(kk[r]);
-      corr[r] = cbias[c] + 128 * wsum[wave_n * WN + 16 * t + 4 * lgrp + r];
-    }
-    const bool k_small = __all(ks);  // wave-uniform precondition of the fast batch-norm form
-#pragma unroll
-    for (int s = 0; s < TM; s++) {
-      const int a0 = acc[t][s][0] + corr[0], a1 = acc[t][s][1] + corr[1];
-      const int a2 = acc[t][s][2] + corr[2], a3 = acc[t][s][3] + corr[3];
-      if constexpr (MODE == EPI_OUT32) {
-        const int m = m0 + wave_m * WM + 16 * s + l16;
-        if (m < g.M) {
-          int *o = (int *)g.out + (long long)m * g.N + n0 + cb + 4 * t;
-          const int v[4] = {a0, a1, a2, a3};
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-            if (n0 + cb + 4 * t + r < g.N) o[r] = v[r];
-        }
-      } else {
-        packed[s][t] = acc24 ? requant4<QM, true>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift)
-                             : requant4<QM, false>(a0, a1, a2, a3, kk, ll, k_small, e.mult, e.shift);
-      }
-    }
-  }
-  if constexpr (MODE != EPI_OUT32) {
-    // one copy of the store code per cache policy
-    auto put = [&](auto nt) {
-      constexpr bool NT = decltype(nt)::value;
-#pragma unroll
-      for (int s = 0; s < TM; s++) {
-        const int m = m0 + wave_m * WM + 16 * s + l16;
-        if (m >= g.M) continue;
-        uint8_t *o = (uint8_t *)g.out + (long long)m * g.N + n0 + cb;
-        if (g.vec_store && n0 + cb + 4 * TN <= g.N) {
-          if constexpr (TN == 4) store16<NT>(o, (v4i){(int)packed[s][0], (int)packed[s][1 % TN], (int)packed[s][2 % TN], (int)packed[s][3 % TN]});
-          else if constexpr (TN == 2) store8<NT>(o, (v2i){(int)packed[s][0], (int)packed[s][1 % TN]});
-          else store4<NT>(o, (int)packed[s][0]);
-        } else {
-#pragma unroll
-          for (int c = 0; c < 4 * TN; c++)
-            if (n0 + cb + c < g.N) o[c] = (uint8_t)(packed[s][c >> 2] >> (8 * (c & 3)));
-        }
-      }
-    };
-    if (g.nt) put(std::true_type{});
-    else put(std::false_type{});
-  }
+  igemm_epilogue<TN, TM, MODE>(acc, g, e, m0, n0, wave_m * WM, wave_n * WN, lane, wsum, cbias, ck_, cl_);
 }

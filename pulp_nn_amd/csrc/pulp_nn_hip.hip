@@ -22,6 +22,7 @@
 #include "calib.h"
 #include "depthwise.h"
 #include "igemm.h"
+#include "igemm_dma.h"
 #include "linear_skinny.h"
 #include "pool.h"
 #include "pw_stream.h"
@@ -112,14 +113,62 @@ void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   }
 }
 
+// Raises a kernel's dynamic-LDS limit above the default 64 KB, once per process and kernel.
+template <auto KERN>
+bool raise_lds_limit(size_t lds)
+{
+  static std::mutex mu;
+  static std::atomic<size_t> limit{65536};
+  if (lds > limit.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (lds > limit.load(std::memory_order_relaxed)) {
+      if (hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+      limit.store(lds, std::memory_order_release);
+    }
+  }
+  return true;
+}
+
+// 256 x 256 tiles fed by LDS-direct loads (igemm_dma.h).  Returns false if the kernel cannot be launched.
+bool launch_igemm_dma(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  g.tiles_n = (g.N + 255) / 256;
+  g.tiles_total = ((g.M + 255) / 256) * g.tiles_n;
+  g.vec_store = (g.N % 16 == 0) && aligned(g.out, 16);
+  g.nt = 0;
+  const size_t lds = (size_t)igd_lds_bytes();
+  const dim3 grid(g.tiles_total), block(IGD_THREADS);
+  switch (mode) {
+    case EPI_BN:
+      if (!raise_lds_limit<igemm_dma_kernel<EPI_BN>>(lds)) return false;
+      hipLaunchKernelGGL(igemm_dma_kernel<EPI_BN>, grid, block, lds, s, g, e);
+      break;
+    case EPI_MULT:
+      if (!raise_lds_limit<igemm_dma_kernel<EPI_MULT>>(lds)) return false;
+      hipLaunchKernelGGL(igemm_dma_kernel<EPI_MULT>, grid, block, lds, s, g, e);
+      break;
+    default:
+      if (!raise_lds_limit<igemm_dma_kernel<EPI_RAW>>(lds)) return false;
+      hipLaunchKernelGGL(igemm_dma_kernel<EPI_RAW>, grid, block, lds, s, g, e);
+      break;
+  }
+  return true;
+}
+
 template <int GATHER>
 void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
   // 256 px x 256 ch with 16 waves when there are at least two such tiles per CU: half the
   // L2 -> LDS bytes per multiply of the 128 x 128 tile
   const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
-  if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
-  else
+  if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) {
+    // whole 128-byte lines per pixel and K slice: operands go HBM/L2 -> LDS without passing through registers
+    if (g.Ci % 128 == 0 && mode != EPI_OUT32 && launch_igemm_dma(mode, g, e, s)) return;
+    launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
+  } else
   // 128 px x 64 ch while 128 x 128 tiles would give a CU at most one workgroup: twice the workgroups to
   // hide each other's latency (such layers are a few K slices long)
   if (g.N > 64 && (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) <= num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);

@@ -1,0 +1,51 @@
+"""GPU parity of the large-tile convolution path (256 x 256 tiles fed by LDS-direct loads).
+
+That path is taken by convolutions with input channels a multiple of 128, more than 128 output channels and
+at least two 256 x 256 tiles per compute unit; these geometries are sized to reach it and to exercise its
+edges (channel tail, pixel tail, padding on every side, stride 2, every epilogue branch, both widths)."""
+import numpy as np
+import pytest
+
+import oracle
+from gpu_helpers import conv, rand_s8, rand_u8, rng_for
+
+pytestmark = pytest.mark.gpu
+
+GEOMS = [
+    # B, H, W, Ci, Co, ky, kx, pads (t, b, l, r), strides
+    (84, 40, 40, 128, 256, 3, 3, (1, 1, 1, 1), (1, 1)),
+    (140, 31, 33, 128, 192, 3, 3, (1, 0, 1, 0), (1, 1)),    # channel tail (192 of a 256 tile), odd sizes, asymmetric pads
+    (150, 60, 62, 128, 136, 3, 3, (0, 1, 0, 1), (2, 2)),    # stride 2, pads bottom / right only
+    (140, 32, 32, 256, 256, 1, 3, (0, 0, 1, 1), (1, 1)),    # 1 x 3 filter, K = 768
+]
+FLAGS = [(1, 1), (1, 0), (0, 0), (0, 1)]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", FLAGS)
+@pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(map(str, g[:7])))
+def test_big_conv(geom, flags, bn_bits):
+    B, H, W, Ci, Co, ky, kx, pads, strides = geom
+    relu, bn = flags
+    r = rng_for(4242 + 3 * relu + bn + bn_bits)
+    x, w, b = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, ky, kx, Ci)), rand_s8(r, (Co,))
+    K = ky * kx * Ci
+    if bn_bits == 64:
+        k, lam, bshift = r.integers(2 ** 20, 2 ** 24, Co), r.integers(-2 ** 36, 2 ** 36, Co), 38 - 3
+    else:
+        k, lam, bshift = r.integers(256, 1025, Co), r.integers(-2 ** 16, 2 ** 16, Co), 20
+    mult = int(r.integers(256, 1025))
+    lg = int(np.log2(K ** 0.5 * 128 * 74))
+    shift = bshift if (relu and bn) else ((lg + 10 - 7) if relu == 1 else max(lg - 7, 0))
+    # the oracle on a sample of the images (whole images: first, last and two in between)
+    sample = sorted({0, B // 3, 2 * B // 3, B - 1})
+    got = conv(x, w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
+    want = oracle.conv(x[sample], w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
+    assert got.shape[1:] == want.shape[1:]
+    assert np.array_equal(got[sample], want), "big conv mismatch"
+    assert want.max() > 0 and (want < 255).any(), "degenerate case"
+    # images are independent: every image with the same input as a checked one must equal it
+    x2 = x.copy()
+    x2[1] = x[0]
+    got2 = conv(x2, w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
+    assert np.array_equal(got2[1], want[0])
