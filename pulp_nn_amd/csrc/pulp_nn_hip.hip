@@ -568,6 +568,39 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
     const dim3 block(64 * DW_WAVES);
+    // whole stride-2 layers with enough tiles to keep a persistent workgroup per compute unit busy: bands
+    // staged by LDS-direct loads, double buffered
+    const int csd_dma = (((g.NR * g.LWD + 3) & ~3)) | 1;  // room for the last 16-byte piece of a band
+    const size_t lds_dma = 2 * (size_t)dwd_buf_dwords(csd_dma) * 4;
+    if (sx == 2 && full && g.CHR == CH && g.B == (int)g_batch && aligned(wt, 4) && (!bias || aligned(bias, 4)) &&
+        (long long)g.B * CH * H * W < 0x7fffffffLL && g.total >= 2 * num_cus() && lds_dma <= 160 * 1024) {
+      const dim3 dgrid(num_cus()), dblock(64 * DWD_WAVES);
+      bool ok = true;
+      g.CSD = csd_dma;
+#define DWD_MODE(S, PL)                                                                                     \
+  switch (mode) {                                                                                           \
+    case EPI_BN:                                                                                            \
+      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_BN>>(lds_dma)))                                 \
+        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_BN>), dgrid, dblock, lds_dma, g_stream, g, e);      \
+      break;                                                                                                \
+    case EPI_MULT:                                                                                          \
+      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_MULT>>(lds_dma)))                               \
+        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_MULT>), dgrid, dblock, lds_dma, g_stream, g, e);    \
+      break;                                                                                                \
+    default:                                                                                                \
+      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_RAW>>(lds_dma)))                                \
+        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_RAW>), dgrid, dblock, lds_dma, g_stream, g, e);     \
+      break;                                                                                                \
+  }
+      if (pl == 1) { DWD_MODE(2, 1) }
+      else { DWD_MODE(2, 0) }
+#undef DWD_MODE
+      if (ok) {
+        check_launch(fn);
+        return;
+      }
+      g.CSD = (g.NR * g.LWD) | 1;
+    }
 #define DW3L_MODE(S, PL, FULL)                                                                                        \
   switch (mode) {                                                                                                     \
     case EPI_BN: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_BN, FULL>), grid, block, ldsl, g_stream, g, e); break;     \

@@ -49,3 +49,47 @@ def test_big_conv(geom, flags, bn_bits):
     x2[1] = x[0]
     got2 = conv(x2, w, b, k, lam, mult, shift, pads, strides, relu, bn, bn_bits)
     assert np.array_equal(got2[1], want[0])
+
+
+# ---- stride-2 depthwise layers large enough for the persistent kernel (bands staged by LDS-direct loads) ----
+# That kernel needs whole 64-channel groups, W % 4 == 0, Wo % 4 == 0 and at least two tiles per compute unit.
+DW_GEOMS = [
+    # B, CH, H, W, pads (t, b, l, r)
+    (130, 128, 56, 56, (1, 1, 1, 1)),    # config 2 geometry: four bands, the top one with a row above the image
+    (520, 64, 30, 32, (1, 0, 1, 0)),     # one band per image, 15 output rows
+    (260, 128, 17, 24, (0, 0, 0, 1)),    # no top / left padding (the other window alignment), 8 x 12 outputs
+    (70, 192, 63, 40, (1, 1, 1, 1)),     # three channel groups, bands of unequal height (32 output rows in 5 bands)
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", [(1, 1), (1, 0), (0, 0)])
+@pytest.mark.parametrize("geom", DW_GEOMS, ids=lambda g: "x".join(map(str, g[:4])))
+def test_big_depthwise_stride2(geom, flags, bn_bits):
+    from gpu_helpers import depthwise_generic
+    B, CH, H, W, pads = geom
+    relu, bn = flags
+    r = rng_for(977 + relu + 2 * bn + bn_bits)
+    x, wt = rand_u8(r, (B, CH, H, W)), rand_s8(r, (CH, 3, 3))
+    b = rand_s8(r, (CH,)) if (relu + bn) % 2 == 0 else None
+    if bn_bits == 64:
+        k, lam, shift = r.integers(2 ** 20, 2 ** 24, CH), r.integers(-2 ** 36, 2 ** 36, CH), 34
+        if bn and relu and CH == 64:
+            k = r.integers(2 ** 33, 2 ** 34, CH)     # k does not fit 32 bits: the general 64-bit path
+            shift = 44
+    else:
+        k, lam, shift = r.integers(2 ** 12, 2 ** 14, CH), r.integers(-2 ** 16, 2 ** 16, CH), 16
+    mult = int(r.integers(256, 1025))
+    if not (relu and bn):
+        shift = 19 if relu == 1 else 9
+    sample = sorted({0, 1, B // 2, B - 1})
+    got = depthwise_generic(x, wt, b, k, lam, mult, shift, pads, (2, 2), relu, bn, bn_bits)
+    want = oracle.depthwise_generic(x[sample], wt, b, k, lam, mult, shift, pads, (2, 2), relu, bn, bn_bits)
+    assert got.shape[1:] == want.shape[1:]
+    assert np.array_equal(got[sample], want), "depthwise mismatch"
+    assert want.max() > 0 and (want < 255).any(), "degenerate case"
+    # a digest over all images against the same layer computed image by image in small batches (other kernel)
+    step = 4
+    parts = [depthwise_generic(x[i:i + step], wt, b, k, lam, mult, shift, pads, (2, 2), relu, bn, bn_bits)
+             for i in range(0, min(B, 24), step)]
+    assert np.array_equal(np.concatenate(parts), got[:min(B, 24)])
