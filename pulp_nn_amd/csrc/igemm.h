@@ -30,14 +30,41 @@
 //     pixel, computed once) ORs the offset to 0xffffffff, which the range check turns
 //     into a load of zeros.  Per K slice that is two VALU instructions per 16-byte chunk
 //     of activations and none per chunk of weights.
+//     With 16 or 32 input channels (GATHER_SUBTAP) a K slice holds four or two whole taps: the
+//     same buffer loads, with the tap of a lane's chunk fixed relative to the slice, so the tap
+//     offset is a handful of VALU instructions per load instead of the general per-chunk
+//     arithmetic (divisions, bounds checks, 64-bit addresses), which is what such small layers
+//     otherwise spend their time on.
 #pragma once
 #include <type_traits>
 
 #include "memops.h"
 #include "requant.h"
 
-enum { GATHER_CHUNK16 = 0, GATHER_BYTES = 1, GATHER_UNIFORM = 2 };
+enum { GATHER_CHUNK16 = 0, GATHER_BYTES = 1, GATHER_UNIFORM = 2, GATHER_SUBTAP = 3 };
 enum { EPI_OUT32 = 3 };  // linear_out_32: int32 accumulators + int32 bias, no requantisation
+
+// Division of a 32-bit unsigned number by a divisor fixed for the launch, as a multiply-high, an add and
+// two shifts (Granlund & Montgomery); the host computes the constants.  The compiler's expansion of a
+// 32-bit division is some 40 instructions, and a tile's set-up divides several times per lane.
+struct FastDiv {
+  unsigned mul, sh1, sh2;
+};
+static inline FastDiv fastdiv_make(unsigned d)
+{
+  FastDiv f;
+  unsigned l = 0;
+  while ((1ull << l) < d) l++;  // ceil(log2(d))
+  f.mul = (unsigned)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+  f.sh1 = l < 1 ? l : 1;
+  f.sh2 = l > 1 ? l - 1 : 0;
+  return f;
+}
+__device__ __forceinline__ unsigned fastdiv(unsigned n, const FastDiv &f)
+{
+  const unsigned t = __umulhi(n, f.mul);
+  return (t + ((n - t) >> f.sh1)) >> f.sh2;
+}
 
 struct ConvGeom {
   const uint8_t *in;
@@ -54,6 +81,10 @@ struct ConvGeom {
   int nt;              // write the output with non-temporal stores
   int tiles_n;         // number of channel tiles
   int tiles_total;     // tiles_m * tiles_n
+  FastDiv d_howo, d_wo, d_tiles_n;  // divisions by HoWo, Wo, tiles_n
+  int batch;           // number of images: ceil(M / HoWo)
+  int ci_shift;        // log2(Ci) when Ci is a power of two (GATHER_SUBTAP), else 0
+  int rkx;             // 65536 / kx + 1: t * rkx >> 16 == t / kx for t < 32 (GATHER_SUBTAP)
 };
 
 #define IGEMM_BK 64
@@ -149,11 +180,16 @@ __device__ __forceinline__ void igemm_epilogue(v4i (&acc)[TN][TM], const ConvGeo
   }
 }
 
-template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4>
+// ONEPASS > 0: the layer has at most ONEPASS K slices and the whole K extent of a tile is staged at
+// once: all global loads of the tile are issued back to back (one memory round trip instead of one
+// per slice), then staged, and after a single barrier the slices are multiplied one after the other.
+// Layers this short are bound by those round trips, not by bytes or multiplies.
+template <int TN, int WAVES_M, int WAVES_N, int GATHER, int MODE, int TM = 4, int ONEPASS = 0>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N,
-                            (WAVES_M * WAVES_N > 8 || TM > 4) ? 1 : (WAVES_M * WAVES_N > 4 || GATHER == GATHER_BYTES ? 2 : IGEMM_MINB))
+                            (WAVES_M * WAVES_N > 8 || TM > 4) ? 1 : (WAVES_M * WAVES_N > 4 || GATHER == GATHER_BYTES || ONEPASS ? 2 : IGEMM_MINB))
 void igemm_kernel(ConvGeom g, EpiArgs e)
 {
+  constexpr int NBUF = ONEPASS ? ONEPASS : 2;  // K slices resident in LDS
   constexpr int WM = 16 * TM, WN = 16 * TN;
   constexpr int BM = WM * WAVES_M, BN = WN * WAVES_N;
   constexpr int NTH = 64 * WAVES_M * WAVES_N;    // threads per workgroup
@@ -162,9 +198,10 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   constexpr int RW = (BN * 4 + NTH - 1) / NTH;   // weight chunks per thread per K slice
   static_assert(BM % RPP == 0, "pixel tile is a whole number of staging passes");
 
-  constexpr bool UNI = GATHER == GATHER_UNIFORM;  // scalar tap walk and buffer loads
-  __shared__ __attribute__((aligned(16))) uint8_t As[2][BM * IGEMM_BK];
-  __shared__ __attribute__((aligned(16))) int8_t Ws[2][BN * IGEMM_BK];
+  constexpr bool SUB = GATHER == GATHER_SUBTAP;                  // several taps per K slice
+  constexpr bool UNI = GATHER == GATHER_UNIFORM || SUB;          // buffer loads with a fixed offset per pixel
+  __shared__ __attribute__((aligned(16))) uint8_t As[NBUF][BM * IGEMM_BK];
+  __shared__ __attribute__((aligned(16))) int8_t Ws[NBUF][BN * IGEMM_BK];
   __shared__ int wsum[BN];
   // per-channel constants of the tile, fetched while the first K slice is on its way
   __shared__ int cbias[BN];
@@ -175,8 +212,9 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   const int wave_m = wave % WAVES_M, wave_n = wave / WAVES_M;
 
   const int tile = xcd_remap(blockIdx.x, g.tiles_total);
-  const int m0 = (tile / g.tiles_n) * BM;
-  const int n0 = (tile % g.tiles_n) * BN;
+  const int tile_m = (int)fastdiv((unsigned)tile, g.d_tiles_n);
+  const int m0 = tile_m * BM;
+  const int n0 = (tile - tile_m * g.tiles_n) * BN;
 
   // ---- per-thread gather state -------------------------------------------
   const int ck = tid & 3;  // which 16-byte chunk of the 64-byte K slice
@@ -186,8 +224,8 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   for (int i = 0; i < RA; i++) {
     const int m = m0 + (tid >> 2) + RPP * i;
     if (m < g.M) {
-      const int b = m / g.HoWo, rem = m - b * g.HoWo;
-      const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
+      const int b = (int)fastdiv((unsigned)m, g.d_howo), rem = m - b * g.HoWo;
+      const int oy = (int)fastdiv((unsigned)rem, g.d_wo), ox = rem - oy * g.Wo;
       iy0[i] = oy * g.sy - g.pt;
       ix0[i] = ox * g.sx - g.pl;
       abase[i] = (long long)b * g.in_img;
@@ -205,7 +243,7 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
   [[maybe_unused]] int u_tap = 0, u_fx = 0, u_fy = 0, u_ci = 0, u_slice = 0;
   if constexpr (UNI) {
     const unsigned shift = (unsigned)((g.pt * g.W + g.pl) * g.Ci);
-    const unsigned batch = (unsigned)((g.M + g.HoWo - 1) / g.HoWo);
+    const unsigned batch = (unsigned)g.batch;
     rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)(g.in - shift), 0, shift + batch * (unsigned)g.in_img, 0x00020000);
     rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)g.w, 0, (unsigned)g.N * (unsigned)g.K, 0x00020000);
 #pragma unroll
@@ -214,9 +252,11 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
       poff[i] = 0xffffffffu;
       pinv[i] = 0;
       if (m < g.M) {
-        const int b = m / g.HoWo, rem = m - b * g.HoWo;
-        const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
-        poff[i] = (unsigned)b * (unsigned)g.in_img + (unsigned)((oy * g.sy * g.W + ox * g.sx) * g.Ci) + 16u * ck;
+        const int b = (int)fastdiv((unsigned)m, g.d_howo), rem = m - b * g.HoWo;
+        const int oy = (int)fastdiv((unsigned)rem, g.d_wo), ox = rem - oy * g.Wo;
+        poff[i] = (unsigned)b * (unsigned)g.in_img + (unsigned)((oy * g.sy * g.W + ox * g.sx) * g.Ci) +
+                  (SUB ? (16u * ck) & (unsigned)(g.Ci - 1) : 16u * ck);
+        if (SUB) pinv[i] = ~0u << (g.kx * g.ky);  // taps past the filter (the tail of the last K slice)
         for (int fy_ = 0, t = 0; fy_ < g.ky; fy_++)
           for (int fx_ = 0; fx_ < g.kx; fx_++, t++) {
             const int iy = oy * g.sy - g.pt + fy_, ix = ox * g.sx - g.pl + fx_;
@@ -225,10 +265,17 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
       }
     }
   }
+  // GATHER_SUBTAP: which of the slice's taps this lane's chunk belongs to, and 65536 / kx rounded up
+  // (t * that >> 16 == t / kx for the tap numbers that occur: t < 32, kx <= 32)
+  [[maybe_unused]] const int sub_h = SUB ? (16 * ck) >> g.ci_shift : 0;
+  [[maybe_unused]] const int sub_rkx = g.rkx;
   // (fy, fx, ci) of byte k = 16*ck of the current K slice
   int kpos = 16 * ck;
-  int ci = kpos % g.Ci, tap = kpos / g.Ci;
-  int fy = tap / g.kx, fx = tap - fy * g.kx;
+  int ci = 0, tap = 0, fy = 0, fx = 0;
+  if constexpr (!UNI) {
+    ci = kpos % g.Ci, tap = kpos / g.Ci;
+    fy = tap / g.kx, fx = tap - fy * g.kx;
+  }
 
   // Weight rows sit in LDS in fragment order: LDS row p = wn*WN + 16*t + i holds
   // channel wn*WN + (i/4)*4*TN + 4*t + (i%4), so that MFMA tile t of a wave reads
@@ -262,12 +309,35 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
     v4i a[RA], w[RW];
     unsigned amask, wmask;  // bit i: chunk i holds real data (else it is staged as zero)
   };
-  Staged R0;
+  [[maybe_unused]] Staged R0;
 
   // Issue the global loads of the next K slice.  Nothing here consumes a loaded value
   // (that would make the wave wait for it): out-of-image taps and out-of-range rows
   // load from a clamped, always valid address and are zeroed when staged into LDS.
   auto gload = [&](Staged &R) {
+    if constexpr (SUB) {
+      typedef unsigned v4u __attribute__((ext_vector_type(4)));
+      // tap of this lane's chunk: taps per slice * slice + (16 * ck) / Ci; at most 31
+      const int t = (u_slice << (6 - g.ci_shift)) + sub_h;
+      const int tfy = (t * sub_rkx) >> 16, tfx = t - tfy * g.kx;
+      const unsigned toff = (unsigned)((tfy * g.W + tfx) * g.Ci);
+#pragma unroll
+      for (int i = 0; i < RA; i++) {
+        const unsigned oob = (unsigned)__builtin_amdgcn_sbfe((int)pinv[i], t, 1);
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (poff[i] + toff) | oob, 0, 0);
+        R.a[i] = (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+      }
+      // weight bytes past the end of a row (K is not a multiple of 64) belong to the next row: out of range instead
+      const unsigned wtail = (u_slice * IGEMM_BK + 16 * ck < g.K) ? 0u : 0xffffffffu;
+#pragma unroll
+      for (int i = 0; i < RW; i++) {
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[i] | wtail, u_slice * IGEMM_BK, 0);
+        R.w[i] = (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+      }
+      R.amask = R.wmask = ~0u;
+      if (u_slice + 1 < KT) u_slice++;
+      return;
+    }
     if constexpr (UNI) {
       typedef unsigned v4u __attribute__((ext_vector_type(4)));
       const int soff_a = (u_fy * g.W + u_fx) * g.Ci + u_ci;  // scalar: tap and channel offset of the slice
@@ -425,15 +495,29 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
       cl_[c] = lv;
     }
   }
-  gload(R0);
-  sts(R0, 0, true);
-  __syncthreads();
-#pragma unroll 1
-  for (int kt = 0; kt < KT; kt++) {
-    gload(R0);                            // slice kt + 1
-    compute(kt & 1);                      // slice kt
-    sts(R0, (kt + 1) & 1, kt + 1 < KT);
+  if constexpr (ONEPASS > 0) {
+    Staged R[ONEPASS];
+#pragma unroll
+    for (int kt = 0; kt < ONEPASS; kt++)
+      if (kt < KT) gload(R[kt]);
+#pragma unroll
+    for (int kt = 0; kt < ONEPASS; kt++)
+      if (kt < KT) sts(R[kt], kt, true);
     __syncthreads();
+#pragma unroll
+    for (int kt = 0; kt < ONEPASS; kt++)
+      if (kt < KT) compute(kt);
+  } else {
+    gload(R0);
+    sts(R0, 0, true);
+    __syncthreads();
+#pragma unroll 1
+    for (int kt = 0; kt < KT; kt++) {
+      gload(R0);                            // slice kt + 1
+      compute(kt & 1);                      // slice kt
+      sts(R0, (kt + 1) & 1, kt + 1 < KT);
+      __syncthreads();
+    }
   }
   // ---- per-row weight sums -> LDS (indexed by LDS row) ---------------------
 #pragma unroll

@@ -50,15 +50,16 @@ __global__ __launch_bounds__(IGD_THREADS, 1) void igemm_dma_kernel(ConvGeom g, E
   const int l16 = lane & 15, lgrp = lane >> 4;
 
   const int tile = xcd_remap(blockIdx.x, g.tiles_total);
-  const int m0 = (tile / g.tiles_n) * BM;
-  const int n0 = (tile % g.tiles_n) * BN;
+  const int tile_m = (int)fastdiv((unsigned)tile, g.d_tiles_n);
+  const int m0 = tile_m * BM;
+  const int n0 = (tile - tile_m * g.tiles_n) * BN;
 
   // ---- what this lane fetches ------------------------------------------------------------------
   // A load instruction of wave w fills LDS rows 16*rb .. 16*rb+15 of one sub-slice, rb = 2*w + j:
   // lane l writes slot l%4 of row 16*rb + l/4, which has to hold K chunk (l%4) ^ ((row/2)%4).
   const unsigned OOB = 0x80000000u;  // offsets stay below 2^31 (checked by the host), so this bit puts a load out of range
   const unsigned shift = (unsigned)((g.pt * g.W + g.pl) * g.Ci);
-  const unsigned batch = (unsigned)((g.M + g.HoWo - 1) / g.HoWo);
+  const unsigned batch = (unsigned)g.batch;
   const __amdgpu_buffer_rsrc_t rsrc_a =
       __builtin_amdgcn_make_buffer_rsrc((void *)(g.in - shift), 0, shift + batch * (unsigned)g.in_img, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_w =
@@ -72,8 +73,8 @@ __global__ __launch_bounds__(IGD_THREADS, 1) void igemm_dma_kernel(ConvGeom g, E
     poff[j] = OOB;
     pinv[j] = 0;
     if (m < g.M) {
-      const int b = m / g.HoWo, rem = m - b * g.HoWo;
-      const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
+      const int b = (int)fastdiv((unsigned)m, g.d_howo), rem = m - b * g.HoWo;
+      const int oy = (int)fastdiv((unsigned)rem, g.d_wo), ox = rem - oy * g.Wo;
       poff[j] = (unsigned)b * (unsigned)g.in_img + (unsigned)((oy * g.sy * g.W + ox * g.sx) * g.Ci) + 16u * chunk;
       for (int fy_ = 0, t = 0; fy_ < g.ky; fy_++)
         for (int fx_ = 0; fx_ < g.kx; fx_++, t++) {

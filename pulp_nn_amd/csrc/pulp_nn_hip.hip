@@ -93,23 +93,36 @@ int num_cus()
 
 // ---- implicit GEMM dispatch -------------------------------------------------
 
-template <int TN, int WM_, int WN_, int GATHER, int TM = 4>
+// launch-constant divisions of the tiled kernels (call after tiles_n is known)
+void conv_geom_divs(ConvGeom &g)
+{
+  g.d_howo = fastdiv_make((unsigned)g.HoWo);
+  g.d_wo = fastdiv_make((unsigned)g.Wo);
+  g.d_tiles_n = fastdiv_make((unsigned)g.tiles_n);
+  g.batch = (g.M + g.HoWo - 1) / g.HoWo;
+  g.ci_shift = 0;
+  while ((1 << (g.ci_shift + 1)) <= g.Ci) g.ci_shift++;
+  g.rkx = 65536 / g.kx + 1;
+}
+
+template <int TN, int WM_, int WN_, int GATHER, int TM = 4, int ONEPASS = 0>
 void launch_igemm_mode(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
   constexpr int BM = 16 * TM * WM_, BN = 16 * TN * WN_;
   const int tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   g.tiles_total = tiles_m * g.tiles_n;
+  conv_geom_divs(g);
   g.vec_store = (g.N % (4 * TN) == 0) && aligned(g.out, 4 * TN);
   // default store policy: the tiled kernel is not bound by HBM, its 16-byte pieces would reach HBM
   // uncombined with the streaming policy (1.36 x the bytes), and the next layer finds the output in cache
   g.nt = 0;
   dim3 grid(g.tiles_total), block(64 * WM_ * WN_);
   switch (mode) {
-    case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN, TM>), grid, block, 0, s, g, e); break;
-    case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT, TM>), grid, block, 0, s, g, e); break;
-    case EPI_RAW: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_RAW, TM>), grid, block, 0, s, g, e); break;
-    default: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_OUT32, TM>), grid, block, 0, s, g, e); break;
+    case EPI_BN: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_BN, TM, ONEPASS>), grid, block, 0, s, g, e); break;
+    case EPI_MULT: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_MULT, TM, ONEPASS>), grid, block, 0, s, g, e); break;
+    case EPI_RAW: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_RAW, TM, ONEPASS>), grid, block, 0, s, g, e); break;
+    default: hipLaunchKernelGGL((igemm_kernel<TN, WM_, WN_, GATHER, EPI_OUT32, TM, ONEPASS>), grid, block, 0, s, g, e); break;
   }
 }
 
@@ -137,6 +150,7 @@ bool launch_igemm_dma(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
   g.tiles_n = (g.N + 255) / 256;
   g.tiles_total = ((g.M + 255) / 256) * g.tiles_n;
+  conv_geom_divs(g);
   g.vec_store = (g.N % 16 == 0) && aligned(g.out, 16);
   g.nt = 0;
   const size_t lds = (size_t)igd_lds_bytes();
@@ -158,6 +172,15 @@ bool launch_igemm_dma(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   return true;
 }
 
+// 128 px x 64 ch tiles, for layers too small to fill the machine with larger ones.  With at most five
+// K slices (K <= 320) a tile's whole K extent fits in LDS and is fetched in one go.
+template <int GATHER>
+void launch_igemm_small(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  if (GATHER != GATHER_BYTES && g.K <= 5 * IGEMM_BK) launch_igemm_mode<2, 2, 2, GATHER, 4, 5>(mode, g, e, s);
+  else launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);
+}
+
 template <int GATHER>
 void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
@@ -171,10 +194,10 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   } else
   // 128 px x 64 ch while 128 x 128 tiles would give a CU at most one workgroup: twice the workgroups to
   // hide each other's latency (such layers are a few K slices long)
-  if (g.N > 64 && (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) <= num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);
+  if (g.N > 64 && (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) <= num_cus()) launch_igemm_small<GATHER>(mode, g, e, s);
   else
   if (g.N > 64) launch_igemm_mode<4, 2, 2, GATHER>(mode, g, e, s);       // 128 px x 128 ch
-  else if (g.N > 32 && (g.M + 255) / 256 < 2 * num_cus()) launch_igemm_mode<2, 2, 2, GATHER>(mode, g, e, s);  // 128 px x 64 ch: more workgroups
+  else if (g.N > 32 && (g.M + 255) / 256 < 2 * num_cus()) launch_igemm_small<GATHER>(mode, g, e, s);  // 128 px x 64 ch: more workgroups
   else if (g.N > 32) launch_igemm_mode<4, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 64 ch
   else if (g.N > 16) launch_igemm_mode<2, 4, 1, GATHER>(mode, g, e, s);  // 256 px x 32 ch
   else launch_igemm_mode<1, 4, 1, GATHER>(mode, g, e, s);                // 256 px x 16 ch
@@ -189,7 +212,13 @@ void launch_igemm(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   const bool uniform = chunk16 && (g.Ci % 64 == 0) && g.kx * g.ky <= 32 &&
                        batch * g.in_img + (long long)(g.pt * g.W + g.pl) * g.Ci < 0x7fffffffLL &&
                        (long long)g.N * g.K < 0x7fffffffLL;
+  // 16 or 32 input channels: two or four whole taps per K slice, same buffer loads (one bit per tap up to
+  // the end of the last slice must fit the 32-bit mask)
+  const bool subtap = chunk16 && (g.Ci == 16 || g.Ci == 32) && g.kx * g.ky + 64 / g.Ci <= 32 && g.kx <= 32 &&
+                      batch * g.in_img + (long long)(g.pt * g.W + g.pl) * g.Ci + (long long)(g.ky * g.W + g.kx) * g.Ci < 0x7fffffffLL &&
+                      (long long)g.N * g.K + 64 < 0x7fffffffLL;
   if (uniform) launch_igemm_tile<GATHER_UNIFORM>(mode, g, e, s);
+  else if (subtap) launch_igemm_tile<GATHER_SUBTAP>(mode, g, e, s);
   else if (chunk16) launch_igemm_tile<GATHER_CHUNK16>(mode, g, e, s);
   else launch_igemm_tile<GATHER_BYTES>(mode, g, e, s);
 }
