@@ -8,16 +8,25 @@ pointwise 1x1 convolution 28x28x128 -> 256 channels at batch 256 (scalar
 multiplier requantisation + ReLU), the configuration the headline metric is
 quoted on.  Inputs are resident in HBM before the timed region; successive steps
 rotate through enough buffer sets (> 256 MB in total) that the Infinity Cache
-cannot hold them.  The last line printed is the JSON record.
+cannot hold them.  A timed region is exactly K steps between two device
+synchronisations; because K steps of a 17 us kernel are far too short to time
+once, the region is repeated (at least 5 times and until 5 ms have been timed)
+and the median is reported.  The last line printed is the JSON record.
 
 Besides the headline workload the record carries, under "layers", the other
 single-layer configurations (3x3 conv at batch 256, depthwise 3x3 stride 1 and 2
-at batch 256, the 64-bit batch-norm 3x3 conv at batch 64), each with its own
-achieved fraction of the int8 MFMA peak and of the HBM bandwidth.
+at batch 256, the 64-bit batch-norm 3x3 conv at batch 64 with its max-pool and
+linear layer) and the whole MobileNet chain, each with its own roofline object.
+
+The process exits with status 1 (and "value": null) if any output differs from
+the CPU oracle.
 """
 import argparse
 import json
+import math
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -26,7 +35,26 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA, op/s
 PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
-HBM_TRAFFIC_CFG1 = int((12728.0 * 2.0 + 50193.0) * 1024)   # measured: FETCH_SIZE 12728.0 KiB x 2.0 + WRITE_SIZE 50193.0 KiB
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_all_layers_hbm_traffic.txt")
+
+
+def profiled_traffic():
+    """HBM bytes per launch from the committed rocprofv3 counter summary (FETCH_SIZE and WRITE_SIZE, scaled by
+    what the same counters read for a plain copy): {(kernel name, grid size): bytes}.  Empty if the file is
+    missing; a kernel that has changed its name since the profile was taken is simply not found."""
+    out = {}
+    if not os.path.exists(TRAFFIC_FILE):
+        return out
+    for line in open(TRAFFIC_FILE):
+        m = re.match(r"^(\S.*?)\s+(\d+)\s+([\d.]+)\s+([\d.]+)\s+(\d+)(?:\s+(\d+)\s+([\d.]+))?\s*$", line)
+        if m:
+            out[(m.group(1).strip(), int(m.group(2)))] = int(m.group(5))
+    return out
+
+
+def traffic_for(table, kernel_prefix):
+    hits = [v for (name, _), v in table.items() if name.startswith(kernel_prefix)]
+    return hits[0] if len(hits) == 1 else None
 
 
 def main():
@@ -50,30 +78,53 @@ def main():
     torch.cuda.set_device(0)
     libs = {32: PulpNN(32), 64: PulpNN(64)}
     for L in libs.values():
-        L.use_torch_stream()
+        L.use_torch_stream()     # the library queues on torch's current stream, which the events below time
+    traffic = profiled_traffic()
+    failures = []
 
     def t(a):
         return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
-    def time_launches(fn, steps, warmup):
-        """fn(i) queues one step on torch's current stream (the library's stream).
-        Returns (wall ms per step, device ms per step from HIP events)."""
+    def time_launches(fn, steps, warmup, min_ms=5.0, min_repeats=5, max_repeats=400):
+        """fn(i) queues one step on torch's current stream (the library's stream).  Times regions of exactly
+        `steps` steps, each between two synchronisations; returns the medians of (wall ms per step, device ms
+        per step from HIP events) and the number of regions."""
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        for i in range(steps):
-            fn(i)
-        e1.record()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+        walls, devs, timed, it = [], [], 0.0, warmup
+        while len(walls) < min_repeats or (timed < min_ms and len(walls) < max_repeats):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            e0.record()
+            for _ in range(steps):
+                fn(it)
+                it += 1
+            e1.record()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            walls.append((t1 - t0) * 1e3 / steps)
+            devs.append(e0.elapsed_time(e1) / steps)
+            timed += e0.elapsed_time(e1)
+        return statistics.median(walls), statistics.median(devs), len(walls)
 
     def rotating(nbytes):
         """How many buffer sets make the rotation exceed the 256 MB Infinity Cache twice over."""
-        return max(2, int(np.ceil(600e6 / nbytes)))
+        return max(2, int(math.ceil(600e6 / nbytes)))
+
+    def roofline(bound, ops, nbytes, dev_ms, kernel):
+        sec = dev_ms * 1e-3
+        r = {"bound": bound, "kernel": kernel}
+        if bound == "mfma":
+            r.update(achieved=round(ops / sec / 1e12, 2), peak=PEAK_INT8_OPS / 1e12, unit="TOP/s (int8, 2 x MAC)",
+                     frac=round(ops / sec / PEAK_INT8_OPS, 4))
+        else:
+            r.update(achieved=round(nbytes / sec / 1e9, 1), peak=PEAK_HBM / 1e9, unit="GB/s",
+                     frac=round(nbytes / sec / PEAK_HBM, 4))
+        r["algorithmic_bytes_per_launch"] = nbytes
+        r["traffic"] = traffic_for(traffic, kernel.split("(")[0].strip())
+        return r
 
     # ---- headline: config 1 -------------------------------------------------
     c1 = workloads.config1(batch=256)
@@ -92,17 +143,19 @@ def main():
         L.pulp_nn_pointwise_HoWo_parallel(xs[j], None, bias, outs[j], w, None, None, c1["out_mult"], c1["out_shift"],
                                           W, H, Ci, W, H, Co, 1, 1, 0, 0, 0, 0, 1, 1, c1["relu"], c1["bn"])
 
-    wall_ms, dev_ms = time_launches(step_c1, args.steps, args.warmup)
+    wall_ms, dev_ms, repeats = time_launches(step_c1, args.steps, args.warmup)
 
-    # parity of what was just computed, on a sample of the batch
+    # parity of what was just computed, on a sample of the batch (the oracle is the checker, outside the timed region)
     import oracle
     nchk = 4
     want = oracle.pointwise(c1["x"][:nchk], c1["w"], c1["bias"], None, None, c1["out_mult"], c1["out_shift"],
                             c1["relu"], c1["bn"], 32)
-    got = outs[(args.steps - 1) % nset][:nchk].cpu().numpy()
-    parity = bool(np.array_equal(got, want))
+    parity = all(bool(np.array_equal(o[:nchk].cpu().numpy(), want)) for o in outs)
+    if not parity:
+        failures.append("configs[1] pointwise")
 
     gops = c1["ops"] / (wall_ms * 1e-3) / 1e9
+    head_kernel = "pw_stream_kernel<4, 2, 4, 1, true, 1, 16>"
     rec = {
         "metric": "int8 GOPS and % int8 MFMA peak per conv layer at batch 256; bit-exact",
         "value": round(gops, 1),
@@ -119,36 +172,42 @@ def main():
         "config": {"workload": "configs[1]: pointwise 1x1 conv 28x28x128 -> 256, batch 256, "
                                "out_mult/out_shift requantisation + ReLU (pulp_nn_pointwise_HoWo_parallel)",
                    "batch": B, "gemm_MxNxK": [B * H * W, Co, Ci], "buffer_sets_rotated": nset},
+        "timed_regions": repeats,
         "images_per_s": round(B / (wall_ms * 1e-3), 1),
         "device_ms_per_step": round(dev_ms, 5),
-        "parity": "bit-exact vs CPU oracle on %d images" % nchk if parity else "MISMATCH vs CPU oracle",
+        "parity": "bit-exact vs CPU oracle on %d images of every buffer set" % nchk if parity else "MISMATCH vs CPU oracle",
         "mfma_frac": round(c1["ops"] / (dev_ms * 1e-3) / PEAK_INT8_OPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "pw_stream_kernel<4, 2, 4, 1, true, 1, 16> (weights-stationary pointwise, scalar-multiplier "
-                      "epilogue)",
+            "kernel": head_kernel + " (weights-stationary pointwise, scalar-multiplier epilogue)",
             "achieved": round(c1["bytes"] / (dev_ms * 1e-3) / 1e9, 1),
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
             "frac": round(c1["bytes"] / (dev_ms * 1e-3) / PEAK_HBM, 4),
             "algorithmic_bytes_per_launch": c1["bytes"],
-            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x 2.0, the factor a plain copy of known
-            # size shows for that counter) and WRITE_SIZE (x 1.0): profiles/bench_all_layers_hbm_traffic.txt
-            "traffic": HBM_TRAFFIC_CFG1,
+            # HBM bytes per launch read at run time from the committed counter summary (rocprofv3 --pmc FETCH_SIZE
+            # x 2.0 + WRITE_SIZE x 1.0, the factors a plain copy of known size shows); null if the file has no
+            # line for this kernel
+            "traffic": traffic_for(traffic, head_kernel),
+            "traffic_source": "profiles/bench_all_layers_hbm_traffic.txt",
         },
     }
 
     # ---- the other single-layer configurations ------------------------------
     layers = []
 
-    def layer_record(name, ops, nbytes, wall, dev, ok):
-        layers.append({
-            "layer": name, "ms": round(dev, 5), "wall_ms": round(wall, 5),
-            "gops": round(ops / (dev * 1e-3) / 1e9, 1),
-            "mfma_frac": round(ops / (dev * 1e-3) / PEAK_INT8_OPS, 4),
-            "hbm_gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
-            "hbm_frac": round(nbytes / (dev * 1e-3) / PEAK_HBM, 4),
-            "parity": "bit-exact" if ok else "MISMATCH"})
+    def layer_record(name, ops, nbytes, wall, dev, ok, bound, kernel, **extra):
+        rec_ = {"layer": name, "ms": round(dev, 5), "wall_ms": round(wall, 5),
+                "gops": round(ops / (dev * 1e-3) / 1e9, 1),
+                "mfma_frac": round(ops / (dev * 1e-3) / PEAK_INT8_OPS, 4),
+                "hbm_gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+                "hbm_frac": round(nbytes / (dev * 1e-3) / PEAK_HBM, 4),
+                "roofline": roofline(bound, ops, nbytes, dev, kernel),
+                "parity": "bit-exact" if ok else "MISMATCH"}
+        rec_.update(extra)
+        layers.append(rec_)
+        if not ok:
+            failures.append(name)
 
     if not args.no_layers:
         steps, warm = max(10, args.steps // 4), max(3, args.warmup // 4)
@@ -168,11 +227,13 @@ def main():
             L.pulp_nn_conv_Ho_parallel(xs0[j], None, b0, outs0[j], w0, k0, l0, 0, c0["out_shift"], 16, 16, 32, 16, 16,
                                        64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
 
-        wall, dev = time_launches(step_c0, steps, warm)
+        wall, dev, _ = time_launches(step_c0, steps, warm)
         want = oracle.conv(c0["x"][:8], c0["w"], c0["bias"], c0["k"], c0["lam"], 0, c0["out_shift"], c0["pads"],
                            c0["strides"], 1, 1, 32)
         layer_record(c0["name"] + "_b256", c0["ops"], c0["bytes"], wall, dev,
-                     np.array_equal(outs0[0][:8].cpu().numpy(), want))
+                     np.array_equal(outs0[0][:8].cpu().numpy(), want), "mfma",
+                     "igemm_kernel<2, 2, 2, 3, 0, 4, 5> (128 x 64 tiles, whole K in one pass)",
+                     note="6.3 MB and 2.4 GOP per launch: bound by launch and memory latency, not by a pipe")
         del xs0, outs0
 
         # config 2: depthwise 3x3, stride 1 through pulp_nn_depthwise_3x3_s1, stride 2 through depthwise_generic
@@ -192,6 +253,7 @@ def main():
                     L.pulp_nn_depthwise_3x3_s1(xs2[j], outs2[j], 58, 56, 128, 1, 1, w2, c2["out_shift"], 0, k2, l2,
                                                1, 1, None)
                 want = oracle.depthwise_3x3_s1(xin[:2], c2["w"], c2["k"], c2["lam"], 0, c2["out_shift"], 1, 1, 1, 1, 32)
+                kern = "dw3x3_lin_kernel<1, 1, 0, true>"
             else:
                 def step_c2(i):
                     j = i % nset
@@ -199,9 +261,10 @@ def main():
                                                 56, 56, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1, 2, 2, 1, 1)
                 want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
                                                 (1, 1, 1, 1), (2, 2), 1, 1, 32)
-            wall, dev = time_launches(step_c2, steps, warm)
+                kern = "dw3x3_dma_kernel<2, 1, 0>"
+            wall, dev, _ = time_launches(step_c2, steps, warm)
             layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev,
-                         np.array_equal(outs2[0][:2].cpu().numpy(), want))
+                         np.array_equal(outs2[0][:2].cpu().numpy(), want), "hbm", kern)
             del xs2, outs2
 
         # config 4: 64-bit batch-norm 3x3 conv at batch 64 (the MFMA-bound layer)
@@ -219,11 +282,15 @@ def main():
             L4.pulp_nn_conv_Ho_parallel(xs4[j], None, b4, outs4[j], w4, k4, l4, 0, c4["out_shift"], 64, 64, 256, 63, 63,
                                         256, 3, 3, 1, 0, 1, 0, 1, 1, 1, 1)
 
-        wall, dev = time_launches(step_c4, max(5, steps // 4), 2)
+        wall, dev, _ = time_launches(step_c4, max(5, steps // 4), 2, min_ms=8.0)
         want = oracle.conv(c4["x"][:1], c4["w"], c4["bias"], c4["k"], c4["lam"], 0, c4["out_shift"], c4["pads"],
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
         layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev,
-                     np.array_equal(outs4[0][:1].cpu().numpy(), want))
+                     np.array_equal(outs4[0][:1].cpu().numpy(), want), "mfma",
+                     "igemm_dma_kernel<0> (256 x 256 tiles, LDS-direct loads)",
+                     note="random int8 operands: the matrix cores alone sustain 3.6-4.0 POP/s on this data "
+                          "(clock drops under the power limit), 2.7-3.0 POP/s with the tile's operand feed from "
+                          "LDS: profiles/mfma_ceiling.txt")
         # the rest of configuration 4: maxpool 2x2 s2 (63 -> 32) and the 1024 -> 4096 linear layer
         pooled = [torch.zeros((64, 32, 32, 256), dtype=torch.uint8, device="cuda") for _ in range(nset)]
 
@@ -231,27 +298,30 @@ def main():
             j = i % nset
             L4.pulp_nn_maxpool(outs4[j], pooled[j], 63, 63, 256, 32, 32, 2, 2, 0, 0, 0, 0, 2, 2)
 
-        wall, dev = time_launches(step_mp, steps, warm)
+        wall, dev, _ = time_launches(step_mp, steps, warm)
         want = oracle.maxpool(outs4[0][:2].cpu().numpy(), (2, 2), (2, 2), out_hw=(32, 32))
         mp_bytes = 64 * (63 * 63 * 256 + 32 * 32 * 256)
         layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev,
-                     np.array_equal(pooled[0][:2].cpu().numpy(), want))
-        vec = torch.randint(0, 255, (64, 1024), dtype=torch.uint8, device="cuda")
+                     np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", "maxpool16_kernel<false>")
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(20244)
+        vec = torch.randint(0, 256, (64, 1024), dtype=torch.uint8, device="cuda", generator=gen)
         lw, lb, lk, ll = t(c4["lin_w"]), t(c4["lin_bias"]), t(c4["lin_k"]), t(c4["lin_lam"])
         lout = torch.zeros((64, 4096), dtype=torch.uint8, device="cuda")
 
         def step_lin(i):
             L4.pulp_nn_linear(vec, lb, lout, lw, lk, ll, 0, c4["lin_shift"], 1024, 4096, 1, 1)
 
-        wall, dev = time_launches(step_lin, steps, warm)
+        wall, dev, _ = time_launches(step_lin, steps, warm)
         want = oracle.linear(vec.cpu().numpy(), c4["lin_w"], c4["lin_bias"], c4["lin_k"], c4["lin_lam"], 0,
                              c4["lin_shift"], 1, 1, 64)
         layer_record("cfg4_linear_1024_4096_b64", 2 * 64 * 1024 * 4096, 64 * (1024 + 4096) + 4096 * 1024 + 4096 * 17,
-                     wall, dev, np.array_equal(lout.cpu().numpy(), want))
+                     wall, dev, np.array_equal(lout.cpu().numpy(), want), "hbm", "linear_skinny_kernel<0>",
+                     note="4.5 MB per launch: bound by launch and memory latency")
         del xs4, outs4, pooled
 
-        # configuration 3: the whole MobileNetV1-0.5 chain at batch 256: 29 launches, the layout change
-        # in front of every depthwise layer fused into it (pulp_nn_hip_depthwise_hwc)
+        # configuration 3: the whole MobileNetV1-0.5 chain at batch 256, the layout change in front of every
+        # depthwise layer fused into it (pulp_nn_hip_depthwise_hwc)
         from pulp_nn_amd import mobilenet
         net = mobilenet.build(256)
         runner = mobilenet.Runner(libs[32], net)
@@ -260,13 +330,16 @@ def main():
         def step_net(i):
             runner.run(x3)
 
-        wall, dev = time_launches(step_net, max(5, steps // 4), 2)
+        wall, dev, _ = time_launches(step_net, max(5, steps // 4), 2, min_ms=8.0)
         libs[32].sync()
         import hashlib
         dig = json.load(open(os.path.join(ROOT, "tests", "golden", "config_digests.json")))["cfg3_b256_logits"]["sha256"]
         ok = hashlib.sha256(runner.logits.cpu().numpy().tobytes()).hexdigest() == dig
+        if not ok:
+            failures.append("cfg3 chain")
         layers.append({"layer": "cfg3_mobilenet_v1_0.5_128x128_b256 (whole chain)", "ms": round(dev, 5),
                        "wall_ms": round(wall, 5), "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
+                       "launches": runner.launches if hasattr(runner, "launches") else None,
                        "images_per_s": round(256 / (wall * 1e-3), 1),
                        "mfma_frac": round(net["ops"] / (dev * 1e-3) / PEAK_INT8_OPS, 4),
                        "parity": "bit-exact (logits digest)" if ok else "MISMATCH"})
@@ -294,7 +367,12 @@ def main():
                       "-march=native, one image row per OpenMP task), %.1f s" % (reps, n_img, el),
             "images_per_s": round(n_img * reps / el, 1)}
 
+    if failures:
+        rec["value"] = None
+        rec["parity_failures"] = failures
     print(json.dumps(rec))
+    if failures:
+        sys.exit(1)
 
 
 if __name__ == "__main__":

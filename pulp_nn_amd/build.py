@@ -38,10 +38,29 @@ def build(bn_bits, verbose=False):
     return out
 
 
+def tool_path():
+    return os.path.join(LIBDIR, "mfma_ceiling")
+
+
+def build_tool(verbose=False):
+    """The matrix-core yardstick (csrc/mfma_ceiling.hip): a stand-alone executable, no part of the libraries."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", os.path.join(CSRC, "mfma_ceiling.hip"), "-o", tool_path()]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout)
+    return tool_path()
+
+
 def build_all(verbose=False):
     from concurrent.futures import ThreadPoolExecutor
-    with ThreadPoolExecutor(2) as ex:
-        return list(ex.map(lambda b: build(b, verbose), (32, 64)))
+    with ThreadPoolExecutor(3) as ex:
+        libs = [ex.submit(build, b, verbose) for b in (32, 64)]
+        tool = ex.submit(build_tool, verbose)
+        return [f.result() for f in libs] + [tool.result()]
 
 
 if __name__ == "__main__":
