@@ -73,6 +73,28 @@ void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bi
                                unsigned short ch, unsigned short dim_im_out_x, unsigned short dim_im_out_y,
                                unsigned short stride, signed char flag_relu, signed char flag_batch_norm);
 
+/* A depthwise 3x3 layer (padding 1 on every side, stride 1 or 2, HWC input as
+ * pulp_nn_hip_depthwise_hwc takes it) and the pointwise layer that follows it, in one launch:
+ * no counterpart in the reference, where the depthwise result goes to memory in HWC
+ * (32bit/src/pulp_nn_depthwise_generic.c:179) and the pointwise layer reads it back
+ * (pulp_nn_pointwise_HoWo_parallel.c:103).  The result is bit for bit that of
+ * pulp_nn_hip_depthwise_hwc followed by pulp_nn_pointwise_HoWo_parallel with the same
+ * parameters (dw_*: the depthwise layer's; pw_*: the pointwise layer's, pw_weight[ch_out][ch]);
+ * the intermediate tensor is never written.  k / lambda arrays are int32_t or int64_t as the
+ * build expects.  Supported: dim_im_in_x in {64, 32, 16, 8} (and 4 with stride 1), ch in
+ * {16, 32} or a multiple of 64 up to 1024, ch_out a multiple of 16, output rows a multiple of
+ * the rows a wave takes at once (2 to 8, times 64 / ch for ch < 64), 16-byte aligned pointwise
+ * weights and output.  Anything else sets PULP_NN_HIP_ERR_UNSUPPORTED and queues nothing:
+ * make the two calls instead. */
+void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_in_x,
+                           unsigned short dim_im_in_y, unsigned short ch, unsigned short dim_im_out_x,
+                           unsigned short dim_im_out_y, unsigned short ch_out, unsigned short stride,
+                           const signed char *dw_wt, const signed char *dw_bias, void *dw_k, void *dw_lambda,
+                           unsigned short dw_out_mult, unsigned short dw_out_shift, signed char dw_flag_relu,
+                           signed char dw_flag_batch_norm, const signed char *pw_weight, const signed char *pw_bias,
+                           void *pw_k, void *pw_lambda, unsigned short pw_out_mult, unsigned short pw_out_shift,
+                           signed char pw_flag_relu, signed char pw_flag_batch_norm);
+
 /* ---- calibration of out_shift -------------------------------------------------------
  * A network that requantises with batch-norm + ReLU chooses, per layer,
  * out_shift = floor(log2(max |acc * k[c]|)) - 7, the maximum taken over the batch, all

@@ -84,6 +84,9 @@ class PulpNN:
         L.pulp_nn_hip_hwc_to_chw.restype = None
         L.pulp_nn_hip_depthwise_hwc.argtypes = [_PTR] * 6 + [_U16] * 8 + [_I8, _I8]
         L.pulp_nn_hip_depthwise_hwc.restype = None
+        L.pulp_nn_hip_dw_pw_hwc.argtypes = ([_PTR] * 2 + [_U16] * 7 + [_PTR] * 4 + [_U16] * 2 + [_I8] * 2 + [_PTR] * 4 +
+                                            [_U16] * 2 + [_I8] * 2)
+        L.pulp_nn_hip_dw_pw_hwc.restype = None
         _U64 = C.c_uint64
         L.pulp_nn_hip_calib_workspace_bytes.argtypes, L.pulp_nn_hip_calib_workspace_bytes.restype = [_U64], _U64
         L.pulp_nn_hip_calib_conv.argtypes = [_PTR] * 4 + [_U16] * 12 + [_PTR, _U64, _PTR]
@@ -144,6 +147,14 @@ class PulpNN:
         PulpNNError (unsupported) for geometries without a fused kernel."""
         self._call("pulp_nn_hip_depthwise_hwc", _ptr(x), _ptr(bias), _ptr(out), _ptr(wt), _ptr(k), _ptr(lam), out_mult,
                    out_shift, dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, stride, flag_relu, flag_batch_norm)
+
+    def dw_pw_hwc(self, x, out, dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, ch_out, stride, dw_wt, dw_bias, dw_k, dw_lam,
+                  dw_mult, dw_shift, dw_relu, dw_bn, pw_w, pw_bias, pw_k, pw_lam, pw_mult, pw_shift, pw_relu, pw_bn):
+        """3x3 depthwise (padding 1, HWC in) and the pointwise layer behind it in one launch.  Raises
+        PulpNNError (unsupported) for geometries without a fused kernel."""
+        self._call("pulp_nn_hip_dw_pw_hwc", _ptr(x), _ptr(out), dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, ch_out, stride,
+                   _ptr(dw_wt), _ptr(dw_bias), _ptr(dw_k), _ptr(dw_lam), dw_mult, dw_shift, dw_relu, dw_bn,
+                   _ptr(pw_w), _ptr(pw_bias), _ptr(pw_k), _ptr(pw_lam), pw_mult, pw_shift, pw_relu, pw_bn)
 
     # -- calibration ---------------------------------------------------------
     def calib_workspace_bytes(self, n_outputs):

@@ -101,11 +101,13 @@ class Runner(network.Runner):
     """The configuration-3 chain on the generic runner.  fused: depthwise layers read the HWC
     output of the previous layer directly (pulp_nn_hip_depthwise_hwc) where the library has a
     kernel for it; otherwise, and with fused=False, the chain is the reference's:
-    pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic."""
+    pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic.  fuse_blocks: a depthwise layer and the
+    pointwise layer behind it run as one launch (pulp_nn_hip_dw_pw_hwc); the depthwise results are
+    then not materialised (self.activations holds stale buffers for them)."""
 
-    def __init__(self, nn, net, fused=True):
+    def __init__(self, nn, net, fused=True, fuse_blocks="auto"):
         self.net = net
-        super().__init__(nn, descriptor(net), (128, 128, 3), net["batch"], fused=fused)
+        super().__init__(nn, descriptor(net), (128, 128, 3), net["batch"], fused=fused, fuse_blocks=fuse_blocks)
         self.logits = self.act["fc"].view(net["batch"], 1000)
         self.activations = [self.act[L["name"]] for L in net["layers"]]
 

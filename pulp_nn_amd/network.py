@@ -13,7 +13,11 @@ produces the tensor called like the layer.  Activations are HWC uint8, batch out
   depthwise     w [C,ky,kx], bias, pads, strides, requantisation.  The tensor it reads is HWC
                 like all others; the runner changes the layout (pulp_nn_hip_hwc_to_chw +
                 pulp_nn_depthwise_generic) or, for 3x3 / padding 1 layers the library has a
-                fused kernel for, calls pulp_nn_hip_depthwise_hwc
+                fused kernel for, calls pulp_nn_hip_depthwise_hwc; if the next layer is a
+                pointwise layer that is the only reader of the depthwise result, the two run
+                as one launch (pulp_nn_hip_dw_pw_hwc) and the depthwise result is not
+                materialised: Runner(..., fuse_blocks=True) for every such pair, False for none,
+                "auto" (the default) for planes up to 16 pixels wide, where it is not slower
   maxpool       kernel (kx,ky), strides, pads, out_hw      -> pulp_nn_maxpool
   avgpool       kernel, strides, pads, out_hw, lam, shift, add, requant -> pulp_nn_avgpool
   add           in = (a, b), m1, m2, shift                 -> pulp_nn_add
@@ -76,10 +80,11 @@ def infer_shapes(layers, input_shape):
 class Runner:
     """Uploads the parameters once, owns the activation buffers and queues the chain."""
 
-    def __init__(self, nn, layers, input_shape, batch, fused=True):
+    def __init__(self, nn, layers, input_shape, batch, fused=True, fuse_blocks="auto"):
         import torch
         self.nn, self.layers, self.batch, self.torch = nn, layers, batch, torch
         self.fused, self.unfused = fused, set()
+        self.fuse_blocks, self.unfused_blocks, self.launches = fuse_blocks, set(), 0
         self.shapes = infer_shapes(layers, input_shape)
         bn_np = np.int64 if nn.bn_bits == 64 else np.int32
 
@@ -182,9 +187,53 @@ class Runner:
         self.nn.set_batch(self.batch)
         tensors = {"input": x}
         out = x
-        for i, L in enumerate(self.layers):
+        self.launches = 0
+        i = 0
+        while i < len(self.layers):
+            L = self.layers[i]
+            if self._block_fusable(i) and self._queue_block(i, tensors):
+                out = tensors[self.layers[i + 1]["name"]] = self.act[self.layers[i + 1]["name"]]
+                i += 2
+                continue
             out = tensors[L["name"]] = self._queue(i, tensors)
+            self.launches += 2 if (L["op"] == "depthwise" and (not self.fused or i in self.unfused)) else 1
+            i += 1
         return out
+
+    # -- depthwise + pointwise as one launch ------------------------------------------------
+    def _block_fusable(self, i):
+        """Layer i is a 3x3 / padding 1 depthwise layer whose only reader is the pointwise layer i + 1."""
+        if not (self.fused and self.fuse_blocks) or i in self.unfused_blocks or i + 1 >= len(self.layers):
+            return False
+        L, N = self.layers[i], self.layers[i + 1]
+        # "auto": only where the single launch is not slower than the two (measured on MI355X at batch 256:
+        # planes up to 16 pixels wide; wider planes keep more of the machine busy as two launches)
+        if self.fuse_blocks == "auto" and self.shapes[L["in"]][1] > 16:
+            return False
+        if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
+            return False
+        sx, sy = L["strides"]
+        if L["w"].shape[1:3] != (3, 3) or tuple(L["pads"]) != (1, 1, 1, 1) or sx != sy:
+            return False
+        readers = [M for M in self.layers if (M["in"] == L["name"] or (M["op"] == "add" and L["name"] in M["in"]))]
+        return len(readers) == 1
+
+    def _queue_block(self, i, tensors):
+        L, P, N, Q, nn = self.layers[i], self.params[i], self.layers[i + 1], self.params[i + 1], self.nn
+        H, W, Cc = self.shapes[L["in"]]
+        Ho, Wo, Co = self.shapes[N["name"]]
+        k1, l1, m1, s1, r1, b1 = self._requant_args(L, P)
+        k2, l2, m2, s2, r2, b2 = self._requant_args(N, Q)
+        try:
+            nn.dw_pw_hwc(tensors[L["in"]], self.act[N["name"]], W, H, Cc, Wo, Ho, Co, L["strides"][0], P["w"], P.get("bias"),
+                         k1, l1, m1, s1, r1, b1, Q["w"], Q.get("bias"), k2, l2, m2, s2, r2, b2)
+        except PulpNNError as err:
+            if err.code != 2:
+                raise
+            self.unfused_blocks.add(i)    # no fused kernel for this geometry
+            return False
+        self.launches += 1
+        return True
 
     # -- calibration ------------------------------------------------------------------------
     def _calib_buffers(self):

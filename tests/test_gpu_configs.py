@@ -74,20 +74,42 @@ def test_config2_depthwise_stride2_batch256():
 def test_config3_mobilenet_batch256():
     net = mobilenet.build(256)
     L = nn(32)
-    runner = mobilenet.Runner(L, net)
     x = torch.from_numpy(net["x"]).cuda()
-    logits = runner.run(x)
+    # two images through the oracle chain, every intermediate layer kept
+    want_logits, want_layers = cfg3_oracle.forward(net, net["x"][:2], keep=True)
+    # 1. every depthwise + pointwise block as one launch: 16 launches, the depthwise results never materialised
+    runner = mobilenet.Runner(L, net, fuse_blocks=True)
+    got = runner.run(x)
     L.sync()
     L.set_batch(1)
-    got = logits.cpu().numpy()
-    # two images through the oracle chain, every intermediate layer compared
-    want_logits, want_layers = cfg3_oracle.forward(net, net["x"][:2], keep=True)
+    got = got.cpu().numpy()
+    assert not runner.unfused_blocks, "blocks without a fused kernel: %s" % sorted(runner.unfused_blocks)
+    assert runner.launches == 16, runner.launches
+    for i, (Ld, w) in enumerate(zip(net["layers"], want_layers)):
+        if Ld["kind"] != "dw":
+            assert_same(runner.activations[i][:2].cpu().numpy(), w, "config 3 layer %s (blocks fused)" % Ld["name"])
+    assert_same(got[:2], want_logits, "config 3 logits (blocks fused)")
+    check_digest("cfg3_b256_logits", got)
+    # 2. one launch per layer (the layout change fused into the depthwise layers): every layer compared
+    runner = mobilenet.Runner(L, net, fuse_blocks=False)
+    got = runner.run(x)
+    L.sync()
+    L.set_batch(1)
+    got = got.cpu().numpy()
+    assert runner.launches == 29, runner.launches
     for i, (Ld, w) in enumerate(zip(net["layers"], want_layers)):
         assert_same(runner.activations[i][:2].cpu().numpy(), w, "config 3 layer %s" % Ld["name"])
     assert_same(got[:2], want_logits, "config 3 logits")
     check_digest("cfg3_b256_logits", got)
     assert not runner.unfused, "depthwise layers without a fused kernel: %s" % sorted(runner.unfused)
-    # the same chain with the layout changes as separate launches (the reference's call sequence)
+    # 3. the runner's default: blocks fused where that is not slower (planes up to 16 pixels wide)
+    auto = mobilenet.Runner(L, net)
+    got3 = auto.run(x)
+    L.sync()
+    L.set_batch(1)
+    assert auto.launches == 20, auto.launches
+    check_digest("cfg3_b256_logits", got3.cpu().numpy())
+    # 4. the same chain with the layout changes as separate launches (the reference's call sequence)
     plain = mobilenet.Runner(L, net, fused=False)
     got2 = plain.run(x)
     L.sync()
