@@ -206,6 +206,8 @@ class Runner:
         if not (self.fused and self.fuse_blocks) or i in self.unfused_blocks or i + 1 >= len(self.layers):
             return False
         L, N = self.layers[i], self.layers[i + 1]
+        if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
+            return False
         # "auto": only where the single launch is not slower than the two (measured on MI355X at batch 256:
         # planes up to 16 pixels wide; wider planes keep more of the machine busy as two launches)
         if self.fuse_blocks == "auto" and self.shapes[L["in"]][1] > 16:
