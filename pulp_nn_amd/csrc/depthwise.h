@@ -141,6 +141,17 @@ __device__ __forceinline__ void dw_tap(const unsigned (&span)[NS], unsigned wA, 
   else acc = __builtin_amdgcn_sdot4((int)dw_window<O, NS>(span), (int)wA, acc, false);
 }
 
+// The first tap of an accumulator: start + K . window.  Asking for the saturating form selects the three-address
+// dot instruction, which takes the start value as an operand of its own; the accumulate-in-place form the compiler
+// otherwise prefers needs a register copy of the start value first.  Nothing here can reach the int32 range
+// (|sum| < 2^21 plus the start value), so saturation never acts.
+template <int O, int NS>
+__device__ __forceinline__ int dw_tap_first(const unsigned (&span)[NS], unsigned wA, unsigned wB, int start)
+{
+  if constexpr (O % 4 == 1) return __builtin_amdgcn_sdot4((int)span[O / 4], (int)wB, start, true);
+  else return __builtin_amdgcn_sdot4((int)dw_window<O, NS>(span), (int)wA, start, true);
+}
+
 // 3x3 depthwise, stride S (1 or 2) in both directions, left padding PL (0 or 1).
 template <int S, int PL, int MODE>
 __global__ __launch_bounds__(256) void dw3x3_kernel(DwGeom g, EpiArgs e)
@@ -254,10 +265,21 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
   bool in_row[NS];
 #pragma unroll
   for (int d = 0; d < NS; d++) in_row[d] = !EDGE || (c.dc0 + d >= 0 && c.dc0 + d < c.LWD);
-  auto read_row = [&](unsigned (&span)[NS]) {
+  // fetch() requests a row's dwords from LDS, finish() turns them into the window bytes; a row is fetched one
+  // step before it is used, so that the LDS latency is covered by the arithmetic of the row before
+  auto fetch = [&](unsigned (&raw)[NS]) {
 #pragma unroll
-    for (int d = 0; d < NS; d++) span[d] = in_row[d] ? (XR ? c.p[d] ^ 0x80808080u : c.p[d]) : 0x80808080u;
+    for (int d = 0; d < NS; d++) raw[d] = in_row[d] ? c.p[d] : (XR ? 0u : 0x80808080u);
     c.p += c.LWD;
+  };
+  auto finish = [&](const unsigned (&raw)[NS], unsigned (&span)[NS]) {
+#pragma unroll
+    for (int d = 0; d < NS; d++) span[d] = XR ? raw[d] ^ 0x80808080u : raw[d];
+  };
+  auto read_row = [&](unsigned (&span)[NS]) {
+    unsigned raw[NS];
+    fetch(raw);
+    finish(raw, span);
   };
   // K_i . window_j of one input row, for the four output columns j
   auto taps = [&](const unsigned (&span)[NS], int i, int (&acc)[4]) {
@@ -265,6 +287,12 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
     dw_tap<O0 + S, NS>(span, c.wA[i], c.wB[i], acc[1]);
     dw_tap<O0 + 2 * S, NS>(span, c.wA[i], c.wB[i], acc[2]);
     dw_tap<O0 + 3 * S, NS>(span, c.wA[i], c.wB[i], acc[3]);
+  };
+  auto taps_first = [&](const unsigned (&span)[NS], int (&acc)[4]) {
+    acc[0] = dw_tap_first<O0, NS>(span, c.wA[0], c.wB[0], c.corr);
+    acc[1] = dw_tap_first<O0 + S, NS>(span, c.wA[0], c.wB[0], c.corr);
+    acc[2] = dw_tap_first<O0 + 2 * S, NS>(span, c.wA[0], c.wB[0], c.corr);
+    acc[3] = dw_tap_first<O0 + 3 * S, NS>(span, c.wA[0], c.wB[0], c.corr);
   };
   auto emit = [&](int (&acc)[4]) {
     unsigned packed = requant4_same<MODE, FASTQ>(acc[0], acc[1], acc[2], acc[3], c.k, c.lambda, c.mult, c.shift);
@@ -286,50 +314,43 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
     // P: output row y-2 so far (K0, K1 rows done); Q: output row y-1 so far (K0 done)
     int P[4], Q[4];
     read_row(span);
-#pragma unroll
-    for (int j = 0; j < 4; j++) P[j] = c.corr;
-    taps(span, 0, P);
+    taps_first(span, P);
     read_row(span);
-#pragma unroll
-    for (int j = 0; j < 4; j++) Q[j] = c.corr;
     taps(span, 1, P);
-    taps(span, 0, Q);
+    taps_first(span, Q);
     // Three accumulator sets take the roles (finishing, middle, starting) in turn; the
     // loop is unrolled by three so that the hand-over costs no register moves.
     int R[4];
-    auto step = [&](int (&fin)[4], int (&mid)[4], int (&beg)[4]) {
-      read_row(span);
+    unsigned nxt[NS];
+    if (c.rows > 0) fetch(nxt);
+    auto step = [&](int (&fin)[4], int (&mid)[4], int (&beg)[4], bool more) {
+      finish(nxt, span);
+      if (more) fetch(nxt);
       taps(span, 2, fin);
       emit(fin);
       taps(span, 1, mid);
-#pragma unroll
-      for (int j = 0; j < 4; j++) beg[j] = c.corr;
-      taps(span, 0, beg);
+      taps_first(span, beg);
     };
     for (int r = 0; c.rows > 0;) {
-      step(P, Q, R);
+      step(P, Q, R, r + 1 < c.rows);
       if (++r >= c.rows) break;
-      step(Q, R, P);
+      step(Q, R, P, r + 1 < c.rows);
       if (++r >= c.rows) break;
-      step(R, P, Q);
+      step(R, P, Q, r + 1 < c.rows);
       if (++r >= c.rows) break;
     }
   } else {
     // Q: next output row so far (K0 row done)
     int Q[4];
     read_row(span);
-#pragma unroll
-    for (int j = 0; j < 4; j++) Q[j] = c.corr;
-    taps(span, 0, Q);
+    taps_first(span, Q);
     for (int r = 0; r < c.rows; r++) {
       read_row(span);
       taps(span, 1, Q);
       read_row(span);
       taps(span, 2, Q);
       emit(Q);
-#pragma unroll
-      for (int j = 0; j < 4; j++) Q[j] = c.corr;
-      taps(span, 0, Q);
+      taps_first(span, Q);
     }
   }
 }
@@ -352,9 +373,14 @@ __device__ __forceinline__ void dw3x3_column(DwColumn c)
 #ifndef DW_WAVES
 #define DW_WAVES 8  // waves per workgroup of dw3x3_lin_kernel
 #endif
-template <int S, int PL, int MODE, bool FULL>
+// DMA (FULL only; the host checks that byte offsets fit 31 bits and that the channel stride leaves room
+// for a band's last 16-byte piece): the band is staged with buffer loads that write LDS directly, one
+// instruction per channel, instead of through registers (no staging registers, no LDS stores with their
+// bank conflicts, no VALU work); LDS then holds raw bytes and the ^ 0x80 is applied as a dword is read.
+template <int S, int PL, int MODE, bool FULL, bool DMA = false>
 __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiArgs e)
 {
+  static_assert(!DMA || FULL, "LDS-direct staging only for whole 64-channel groups");
   constexpr int NWV = DW_WAVES, CPW = DW_CG / NWV;  // waves, channels staged per wave
   extern __shared__ unsigned dw_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -376,7 +402,38 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
   const int r_lo = max(0, -iy_start), r_hi = min(g.NR, g.H - iy_start);  // rows of the band inside the image
   const int run_len = max(r_hi - r_lo, 0) * g.W;                        // bytes per channel
   const bool two = run_len + 12 > 64 * 16;  // a run may need more than 64 chunks
-  {
+  if constexpr (DMA) {
+    // Lane l fetches the 16-byte chunk l of a channel's band (dwords 4l .. 4l+3).  Dwords [lo_d, hi_d) lie inside
+    // the image; a chunk wholly outside is requested out of range (zeros); a chunk that straddles the first or last
+    // image row is left out and fetched dword by dword (runs of 64 dwords q1 / q2).
+    typedef __attribute__((address_space(3))) void *lds_ptr_t;
+    const unsigned OOB = 0x80000000u;
+    const __amdgpu_buffer_rsrc_t rsrc_in =
+        __builtin_amdgcn_make_buffer_rsrc((void *)g.in, 0, (unsigned)(g.planes * g.H * g.W), 0x00020000);
+    const int nchunks = (g.NR * LWD + 3) >> 2;
+    const int lo_d = r_lo * LWD, hi_d = r_hi * LWD;
+    const int hi_e = r_hi == g.NR ? 0x7fffffff : hi_d;  // nothing to zero behind the last row of the band
+    const int d0 = 4 * lane;
+    const bool inside = d0 >= lo_d && d0 + 3 < hi_e, outside = d0 + 3 < lo_d || d0 >= hi_e;
+    const bool act4 = lane < nchunks && (inside || outside);
+    const unsigned voff4 = inside ? (unsigned)(16 * lane + iy_start * g.W) : OOB;
+    const int q1 = (lo_d & 3) ? (lo_d >> 6) : -1, q2 = (r_hi < g.NR && (hi_d & 3)) ? (hi_d >> 6) : -1;
+    auto fix = [&](unsigned *dst, int soff, int q) {
+      const int d = 64 * q + lane;
+      const bool mine = ((d >> 2) == (lo_d >> 2) && (lo_d & 3)) || ((d >> 2) == (hi_d >> 2) && r_hi < g.NR && (hi_d & 3));
+      const unsigned voff = (d >= lo_d && d < hi_d) ? (unsigned)(4 * d + iy_start * g.W) : OOB;
+      if (mine) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)(dst + 64 * q), 4, (int)voff, soff, 0, 0);
+    };
+#pragma unroll 1
+    for (int cc = 0; cc < CPW; cc++) {
+      const int c = wave + NWV * cc;
+      const int soff = ((b * g.CH + c0 + c) * g.H) * g.W;
+      unsigned *dst = dw_lds + c * g.CSD;
+      if (act4) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)dst, 16, (int)voff4, soff, 0, 0);
+      if (q1 >= 0) fix(dst, soff, q1);
+      if (q2 >= 0 && q2 != q1) fix(dst, soff, q2);
+    }
+  } else {
     v4i ld[CPW][2];
     int mis[CPW];
 #pragma unroll
@@ -438,6 +495,7 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
     for (int i = 0; i < 3; i++) wA[i] = wB[i] = 0;
   }
   const bool k_small = __all(bn_k_small(kk));
+  if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's LDS-direct loads have landed
   __syncthreads();
 
   // ---- compute -------------------------------------------------------------------------
@@ -475,11 +533,11 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
     col.nbytes = (int)min(4ll, max(left, 0ll));
     const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
     if (fastq) {
-      if (edge) dw3x3_column<S, PL, MODE, FULL, true, true>(col);
-      else dw3x3_column<S, PL, MODE, FULL, false, true>(col);
+      if (edge) dw3x3_column<S, PL, MODE, FULL, true, true, DMA>(col);
+      else dw3x3_column<S, PL, MODE, FULL, false, true, DMA>(col);
     } else {
-      if (edge) dw3x3_column<S, PL, MODE, FULL, true, false>(col);
-      else dw3x3_column<S, PL, MODE, FULL, false, false>(col);
+      if (edge) dw3x3_column<S, PL, MODE, FULL, true, false, DMA>(col);
+      else dw3x3_column<S, PL, MODE, FULL, false, false, DMA>(col);
     }
   }
 }

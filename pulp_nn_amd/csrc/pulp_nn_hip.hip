@@ -505,7 +505,13 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     g.LP = 0;
     g.LWD = W / 4;
   }
-  const int max_csd = 255;  // 64 channels x 255 dwords = 63.75 KiB of LDS
+  int max_csd = 255;  // 64 channels x 255 dwords = 63.75 KiB of LDS
+  // Stride 1 on whole 64-channel groups (the LDS-direct staging of dw3x3_lin_kernel): bands of under 40 KiB, so that
+  // four workgroups share a compute unit and the loads of one are covered by the arithmetic of the others; not
+  // when that would leave fewer than 6 output rows per band (two more input rows are staged than rows come out).
+  const bool lin_dma_ok = lin && CH % DW_CG == 0 && Wo % 4 == 0 && aligned(out, 4) &&
+                          (long long)g_batch * CH * H * W < 0x7fffffffLL;
+  if (lin_dma_ok && sx == 1 && 156 / g.LWD - ky + 1 >= 6) max_csd = 156;
   int nr_max = max_csd / g.LWD;
   if (nr_max < ky) return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "image too wide for the LDS tile");
   int rb_max = (nr_max - ky) / sy + 1;
@@ -637,17 +643,30 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     case EPI_MULT: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_MULT, FULL>), grid, block, ldsl, g_stream, g, e); break; \
     default: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_RAW, FULL>), grid, block, ldsl, g_stream, g, e); break;        \
   }
+#define DW3L_DMA(S, PL)                                                                                                     \
+  switch (mode) {                                                                                                           \
+    case EPI_BN: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_BN, true, true>), grid, block, ldsd, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_MULT, true, true>), grid, block, ldsd, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_RAW, true, true>), grid, block, ldsd, g_stream, g, e); break;        \
+  }
 #define DW3L(S, PL)          \
-  if (full) {                \
+  if (full && lin_dma) {     \
+    DW3L_DMA(S, PL)          \
+  } else if (full) {         \
     DW3L_MODE(S, PL, true)   \
   } else {                   \
     DW3L_MODE(S, PL, false)  \
   }
+    // whole 64-channel groups: the band staged by LDS-direct loads (the channel stride leaves room for the last piece)
+    const bool lin_dma = full && lin_dma_ok && g.CHR == CH && g.B == (int)g_batch && DW_CG * (size_t)csd_dma * 4 + 16 <= 64 * 1024;
+    const size_t ldsd = DW_CG * (size_t)csd_dma * 4 + 16;
+    if (lin_dma) g.CSD = csd_dma;
     if (sx == 1 && pl == 1) { DW3L(1, 1) }
     else if (sx == 1) { DW3L(1, 0) }
     else if (pl == 1) { DW3L(2, 1) }
     else { DW3L(2, 0) }
 #undef DW3L
+#undef DW3L_DMA
 #undef DW3L_MODE
   } else if (fast) {
     if (sx == 1 && pl == 1) { switch (mode) {

@@ -93,3 +93,38 @@ def test_big_depthwise_stride2(geom, flags, bn_bits):
     parts = [depthwise_generic(x[i:i + step], wt, b, k, lam, mult, shift, pads, (2, 2), relu, bn, bn_bits)
              for i in range(0, min(B, 24), step)]
     assert np.array_equal(np.concatenate(parts), got[:min(B, 24)])
+
+
+# ---- stride-1 depthwise on whole 64-channel groups: bands staged by LDS-direct loads in the band kernel ----
+DW1_GEOMS = [
+    # B, CH, H, W, pads (t, b, l, r)
+    (6, 128, 56, 56, (1, 1, 1, 1)),      # config 2 geometry: seven bands of eight output rows
+    (5, 64, 20, 20, (1, 1, 1, 1)),       # rows of 5 dwords: the 16-byte pieces straddle the image's first and last row
+    (4, 192, 45, 24, (0, 1, 0, 2)),      # no top / left padding, two bands, three channel groups
+    (3, 64, 9, 112, (1, 1, 1, 1)),       # wide rows: the 64 KiB band limit applies instead of the 40 KiB one
+    (2, 64, 6, 8, (1, 1, 1, 1)),         # a band shorter than one load instruction covers
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", [(1, 1), (1, 0), (0, 0)])
+@pytest.mark.parametrize("geom", DW1_GEOMS, ids=lambda g: "x".join(map(str, g[:4])))
+def test_depthwise_stride1_whole_groups(geom, flags, bn_bits):
+    from gpu_helpers import depthwise_generic
+    B, CH, H, W, pads = geom
+    relu, bn = flags
+    r = rng_for(1977 + relu + 2 * bn + bn_bits)
+    x, wt = rand_u8(r, (B, CH, H, W)), rand_s8(r, (CH, 3, 3))
+    b = rand_s8(r, (CH,)) if (relu + bn) % 2 == 0 else None
+    if bn_bits == 64:
+        k, lam, shift = r.integers(2 ** 20, 2 ** 24, CH), r.integers(-2 ** 36, 2 ** 36, CH), 34
+    else:
+        k, lam, shift = r.integers(2 ** 12, 2 ** 14, CH), r.integers(-2 ** 16, 2 ** 16, CH), 16
+    mult = int(r.integers(256, 1025))
+    if not (relu and bn):
+        shift = 19 if relu == 1 else 9
+    got = depthwise_generic(x, wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
+    want = oracle.depthwise_generic(x, wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want), "depthwise mismatch"
+    assert want.max() > 0 and (want < 255).any(), "degenerate case"
