@@ -253,7 +253,7 @@ def main():
                     L.pulp_nn_depthwise_3x3_s1(xs2[j], outs2[j], 58, 56, 128, 1, 1, w2, c2["out_shift"], 0, k2, l2,
                                                1, 1, None)
                 want = oracle.depthwise_3x3_s1(xin[:2], c2["w"], c2["k"], c2["lam"], 0, c2["out_shift"], 1, 1, 1, 1, 32)
-                kern = "dw3x3_lin_kernel<1, 1, 0, true>"
+                kern = "dw3x3_lin_kernel<1, 1, 0, true, true>"
             else:
                 def step_c2(i):
                     j = i % nset
@@ -261,7 +261,7 @@ def main():
                                                 56, 56, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1, 2, 2, 1, 1)
                 want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
                                                 (1, 1, 1, 1), (2, 2), 1, 1, 32)
-                kern = "dw3x3_dma_kernel<2, 1, 0>"
+                kern = "dw3x3_lin_kernel<2, 1, 0, true, true>"
             wall, dev, _ = time_launches(step_c2, steps, warm)
             layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev,
                          np.array_equal(outs2[0][:2].cpu().numpy(), want), "hbm", kern)

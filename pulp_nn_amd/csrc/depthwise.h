@@ -255,8 +255,8 @@ struct DwColumn {
   int store, nbytes;
 };
 
-// XR: LDS holds the raw input bytes and the ^ 0x80 is applied as a dword is read (the staging of
-// dw3x3_dma_kernel cannot apply it).
+// XR: LDS holds the raw input bytes and the ^ 0x80 is applied as a dword is read (the LDS-direct staging of
+// dw3x3_lin_kernel cannot apply it).
 template <int S, int PL, int MODE, bool FULL, bool EDGE, bool FASTQ, bool XR = false>
 __device__ __forceinline__ void dw3x3_column(DwColumn c)
 {
@@ -538,202 +538,6 @@ __global__ __launch_bounds__(64 * DW_WAVES) void dw3x3_lin_kernel(DwGeom g, EpiA
     } else {
       if (edge) dw3x3_column<S, PL, MODE, FULL, true, false, DMA>(col);
       else dw3x3_column<S, PL, MODE, FULL, false, false, DMA>(col);
-    }
-  }
-}
-
-// 3x3 depthwise, stride 2, for whole layers of 64-channel groups (the FULL case of dw3x3_lin_kernel),
-// persistent:
-// one workgroup per compute unit works through a contiguous run of tiles (tile = image x 64 channels x
-// band of output rows, as in dw3x3_lin_kernel) with two LDS buffers.  The band of tile k+1 travels
-// HBM -> LDS with buffer loads that write LDS directly (buffer_load_dword ... lds: no registers, no
-// LDS store instructions, no VALU work) while tile k is computed, so the memory system always has a
-// tile's worth of requests from every compute unit and the arithmetic waves keep their issue slots.
-// Such a load writes 64 consecutive 16-byte pieces of LDS (lane l at 16*l; neither side needs more
-// than dword alignment): a channel's band (rows contiguous in its CHW plane, at most 1 KB) is one
-// instruction.  (With one dword per lane a band takes four, and these instructions issue at a fixed
-// rate of about 25 cycles each: 3 us per tile.)  Rows of the band above or below the image are
-// requested out of range, which writes zeros; LDS holds raw bytes and the ^ 0x80 is applied when a
-// dword is read (zero -> 0x80, the value of padding).  The channel stride in LDS leaves room for the
-// last piece when the band is not a whole number of them.  The per-channel constants of a tile
-// (weights, bias, k, lambda of its 64 channels) take the same road into a small LDS area behind the
-// band, so that the computing waves execute no load at all and never wait for their output stores.
-// The kernel is bound by the vector ALU (the arithmetic of a tile takes longer than its bytes): it
-// is used for stride 2 (config 2: 36 us against 39 us for dw3x3_lin_kernel); at stride 1, with four
-// times the outputs per input byte, two resident workgroups of dw3x3_lin_kernel share the ALU
-// better than one persistent workgroup of 16 waves (64 us against 74 us), so stride 1 stays there.
-#define DWD_WAVES 16
-#define DWD_CONST_DW (144 + 16 + 2 * 64 * (int)(sizeof(bn_t) / 4))  // weights, bias, k, lambda (dwords)
-__host__ __device__ static inline int dwd_buf_dwords(int csd) { return DW_CG * csd + DWD_CONST_DW; }
-
-template <int S, int PL, int MODE>
-__global__ __launch_bounds__(64 * DWD_WAVES) void dw3x3_dma_kernel(DwGeom g, EpiArgs e)
-{
-  typedef __attribute__((address_space(3))) void *lds_ptr_t;
-  extern __shared__ unsigned dw_lds[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int LWD = g.LWD;                       // = W / 4
-  const int nchunks = (g.NR * LWD + 3) >> 2;   // 16-byte chunks of a channel's band (at most 64: the band is at most 255 dwords)
-  const int bufd = dwd_buf_dwords(g.CSD);
-  const unsigned OOB = 0x80000000u;            // byte offsets stay below 2^31 (checked by the host)
-
-  // this workgroup's run of tiles
-  const int v = dw_xcd_remap(blockIdx.x, gridDim.x);
-  const int t_beg = (int)((long long)g.total * v / gridDim.x);
-  const int t_end = (int)((long long)g.total * (v + 1) / gridDim.x);
-
-  // Which waves issue the requests: the ones that have no column group to compute (the 14 groups of a
-  // 56-pixel row leave two of the 16 waves free), all of them when every wave computes.  A wave that
-  // computes would issue its requests behind the output stores still queued in the compute unit's
-  // memory pipeline and stand still for a microsecond or two.
-  const int xg_n = g.Wo >> 2;
-  const int rq_n = xg_n < DWD_WAVES ? DWD_WAVES - xg_n : DWD_WAVES;
-  const bool requester = xg_n < DWD_WAVES ? wave >= xg_n : true;
-  const int rq_id = xg_n < DWD_WAVES ? wave - xg_n : wave;
-
-  const __amdgpu_buffer_rsrc_t rsrc_in =
-      __builtin_amdgcn_make_buffer_rsrc((void *)g.in, 0, (unsigned)((long long)g.B * g.CH * g.H * g.W), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_wt = __builtin_amdgcn_make_buffer_rsrc((void *)g.wt, 0, (unsigned)g.CH * 9u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)g.bias, 0, g.bias ? (unsigned)g.CH : 0u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_k =
-      __builtin_amdgcn_make_buffer_rsrc((void *)e.k, 0, MODE == EPI_BN ? (unsigned)g.CH * (unsigned)sizeof(bn_t) : 0u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_l =
-      __builtin_amdgcn_make_buffer_rsrc((void *)e.lambda, 0, MODE == EPI_BN ? (unsigned)g.CH * (unsigned)sizeof(bn_t) : 0u, 0x00020000);
-
-  struct Tile {
-    int c0, oy0, rows, iy_start, b;
-  };
-  auto decode = [&](int t) {
-    Tile T;
-    const int cg = t % g.cgroups;
-    t /= g.cgroups;
-    const int band = t % g.bands;
-    T.b = t / g.bands;
-    T.c0 = cg * DW_CG;
-    T.oy0 = band * g.RB;
-    T.rows = min(g.RB, g.Ho - T.oy0);
-    T.iy_start = T.oy0 * S - g.pt;
-    return T;
-  };
-  // request the band and the constants of tile t into buffer buf
-  auto request = [&](int t, int buf) {
-    const Tile T = decode(t);
-    unsigned *base = dw_lds + buf * bufd;
-    const int r_lo = max(0, -T.iy_start), r_hi = min(g.NR, g.H - T.iy_start);  // rows of the band inside the image
-    // dwords [lo_d, hi_d) of a channel's band lie inside the image.  Lane l fetches the 16-byte chunk
-    // l (dwords 4l .. 4l+3).  A chunk wholly outside is requested out of range (zeros); a chunk
-    // that straddles the first or last image row (only possible in the top and bottom bands, when a
-    // row is not a whole number of chunks) is left out here and fetched dword by dword below.
-    const int lo_d = r_lo * LWD, hi_d = r_hi * LWD;
-    const int hi_e = r_hi == g.NR ? 0x7fffffff : hi_d;  // nothing to zero behind the last row of the band
-    const int d0 = 4 * lane;
-    const bool inside = d0 >= lo_d && d0 + 3 < hi_e, outside = d0 + 3 < lo_d || d0 >= hi_e;
-    const bool act4 = lane < nchunks && (inside || outside);
-    const unsigned voff4 = inside ? (unsigned)(16 * lane + T.iy_start * g.W) : OOB;
-    // the (at most two) straddling chunks, as runs of 64 dwords: run q1 holds dword lo_d - 1 (if lo_d is
-    // not on a chunk boundary), run q2 dword hi_d
-    const int q1 = (lo_d & 3) ? (lo_d >> 6) : -1, q2 = (r_hi < g.NR && (hi_d & 3)) ? (hi_d >> 6) : -1;
-    auto fix = [&](unsigned *dst, int soff, int q) {
-      const int d = 64 * q + lane;
-      const bool mine = ((d >> 2) == (lo_d >> 2) && (lo_d & 3)) || ((d >> 2) == (hi_d >> 2) && r_hi < g.NR && (hi_d & 3));
-      const unsigned voff = (d >= lo_d && d < hi_d) ? (unsigned)(4 * d + T.iy_start * g.W) : OOB;
-      if (mine) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)(dst + 64 * q), 4, (int)voff, soff, 0, 0);
-    };
-#pragma unroll 1
-    for (int c = rq_id; c < DW_CG; c += rq_n) {
-      const int soff = ((T.b * g.CH + T.c0 + c) * g.H) * g.W;
-      unsigned *dst = base + c * g.CSD;
-      if (act4) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)dst, 16, (int)voff4, soff, 0, 0);
-      if (q1 >= 0) fix(dst, soff, q1);
-      if (q2 >= 0 && q2 != q1) fix(dst, soff, q2);
-    }
-    // constants: weights 64 x 9 bytes = 144 dwords, bias 16 dwords, k and lambda 64 values each
-    unsigned *cst = base + DW_CG * g.CSD;
-    // the four pieces go to four requesting waves, or all to the first if there are fewer
-    auto mine = [&](int i) { return rq_n >= 4 ? rq_id == i : rq_id == 0; };
-    if (mine(0)) {
-#pragma unroll
-      for (int q = 0; q < 3; q++)
-        if (64 * q + lane < 144)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_wt, (lds_ptr_t)(cst + 64 * q), 4, 4 * (64 * q + lane), T.c0 * 9, 0, 0);
-    }
-    if (mine(1)) {
-      if (lane < 16) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(cst + 144), 4, 4 * lane, T.c0, 0, 0);
-    }
-    if (MODE == EPI_BN) {
-      constexpr int NQ = (int)sizeof(bn_t) / 4;  // runs of 64 dwords
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-        if (mine(2 + i)) {
-#pragma unroll
-          for (int q = 0; q < NQ; q++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(i == 0 ? rsrc_k : rsrc_l, (lds_ptr_t)(cst + 160 + i * 64 * NQ + 64 * q), 4,
-                                                     4 * (64 * q + lane), T.c0 * (int)sizeof(bn_t), 0, 0);
-        }
-    }
-  };
-
-  const int xgroups = g.Wo >> 2;
-  const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
-  const int cq = lane & ~3;
-  constexpr int NS = ((4 - PL) + 3 * S + 2) / 4 + 1;
-
-  if (requester && t_beg < t_end) request(t_beg, 0);
-#pragma unroll 1
-  for (int t = t_beg; t < t_end; t++) {
-    const int buf = (t - t_beg) & 1;
-    // a requesting wave's loads of tile t have landed (a wave that requests and computes also waits for its
-    // output stores of the tile before: vector memory operations complete in order) ...
-    if (requester) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __builtin_amdgcn_s_barrier();  // ... everybody's have, and everybody has finished reading the other buffer
-    if (requester && t + 1 < t_end) request(t + 1, buf ^ 1);
-
-    const Tile T = decode(t);
-    const unsigned *band = dw_lds + buf * bufd;
-    const unsigned char *cst = (const unsigned char *)(band + DW_CG * g.CSD);
-    // ---- per-lane channel constants (LDS) ---------------------------------------------------------
-    DwColumn col;
-    int wsum = 0;
-#pragma unroll
-    for (int i = 0; i < 3; i++) {
-      const unsigned k0 = cst[lane * 9 + 3 * i], k1 = cst[lane * 9 + 3 * i + 1], k2 = cst[lane * 9 + 3 * i + 2];
-      col.wA[i] = k0 | (k1 << 8) | (k2 << 16);
-      col.wB[i] = col.wA[i] << 8;
-      wsum += (int)(int8_t)k0 + (int)(int8_t)k1 + (int)(int8_t)k2;
-    }
-    col.corr = 128 * wsum + (int)(int8_t)cst[4 * 144 + lane];  // (no bias: the area holds zeros)
-    col.k = col.lambda = 0;
-    if (MODE == EPI_BN) {
-      col.k = ((const bn_t *)(cst + 4 * 160))[lane];
-      col.lambda = ((const bn_t *)(cst + 4 * 160))[64 + lane];
-    }
-    const bool k_small = __all(bn_k_small(col.k));
-    const bool fastq = (MODE == EPI_BN) ? k_small : (e.shift >= 16);
-    col.LWD = LWD;
-    col.rows = T.rows;
-    col.row_bytes = (long long)g.Wo * g.CH;
-    col.mult = e.mult;
-    col.shift = e.shift;
-    col.sel1 = sel1;
-    col.sel2 = sel2;
-    col.store = 0;
-    col.nbytes = 4;
-    const unsigned *lbase = band + lane * g.CSD - 1;
-    uint8_t *obase = g.out + ((((long long)T.b * g.Ho + T.oy0) * g.Wo + (lane & 3)) * g.CH + T.c0 + cq);
-    // ---- compute ---------------------------------------------------------------------------------
-    for (int xg = wave; xg < xgroups; xg += DWD_WAVES) {
-      col.dc0 = xg * S - 1;
-      col.p = lbase + xg * S;
-      col.o = obase + (long long)(4 * xg) * g.CH;
-      const bool edge = col.dc0 < 0 || col.dc0 + NS > LWD;
-      if (fastq) {
-        if (edge) dw3x3_column<S, PL, MODE, true, true, true, true>(col);
-        else dw3x3_column<S, PL, MODE, true, false, true, true>(col);
-      } else {
-        if (edge) dw3x3_column<S, PL, MODE, true, true, false, true>(col);
-        else dw3x3_column<S, PL, MODE, true, false, false, true>(col);
-      }
     }
   }
 }

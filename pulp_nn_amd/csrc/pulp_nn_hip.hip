@@ -506,12 +506,13 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     g.LWD = W / 4;
   }
   int max_csd = 255;  // 64 channels x 255 dwords = 63.75 KiB of LDS
-  // Stride 1 on whole 64-channel groups (the LDS-direct staging of dw3x3_lin_kernel): bands of under 40 KiB, so that
-  // four workgroups share a compute unit and the loads of one are covered by the arithmetic of the others; not
-  // when that would leave fewer than 6 output rows per band (two more input rows are staged than rows come out).
+  // Whole 64-channel groups (the LDS-direct staging of dw3x3_lin_kernel): bands of under 40 KiB, so that four
+  // workgroups share a compute unit and the loads of one are covered by the arithmetic of the others; not when
+  // that would leave fewer than 6 (stride 2: 4) output rows per band (ky - sy more input rows are staged per
+  // band than it consumes alone).
   const bool lin_dma_ok = lin && CH % DW_CG == 0 && Wo % 4 == 0 && aligned(out, 4) &&
                           (long long)g_batch * CH * H * W < 0x7fffffffLL;
-  if (lin_dma_ok && sx == 1 && 156 / g.LWD - ky + 1 >= 6) max_csd = 156;
+  if (lin_dma_ok && (156 / g.LWD - ky) / sy + 1 >= (sx == 1 ? 6 : 4)) max_csd = 156;
   int nr_max = max_csd / g.LWD;
   if (nr_max < ky) return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "image too wide for the LDS tile");
   int rb_max = (nr_max - ky) / sy + 1;
@@ -604,39 +605,7 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
     const dim3 block(64 * DW_WAVES);
-    // whole stride-2 layers with enough tiles to keep a persistent workgroup per compute unit busy: bands
-    // staged by LDS-direct loads, double buffered
     const int csd_dma = (((g.NR * g.LWD + 3) & ~3)) | 1;  // room for the last 16-byte piece of a band
-    const size_t lds_dma = 2 * (size_t)dwd_buf_dwords(csd_dma) * 4;
-    if (sx == 2 && full && g.CHR == CH && g.B == (int)g_batch && aligned(wt, 4) && (!bias || aligned(bias, 4)) &&
-        (long long)g.B * CH * H * W < 0x7fffffffLL && g.total >= 2 * num_cus() && lds_dma <= 160 * 1024) {
-      const dim3 dgrid(num_cus()), dblock(64 * DWD_WAVES);
-      bool ok = true;
-      g.CSD = csd_dma;
-#define DWD_MODE(S, PL)                                                                                     \
-  switch (mode) {                                                                                           \
-    case EPI_BN:                                                                                            \
-      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_BN>>(lds_dma)))                                 \
-        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_BN>), dgrid, dblock, lds_dma, g_stream, g, e);      \
-      break;                                                                                                \
-    case EPI_MULT:                                                                                          \
-      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_MULT>>(lds_dma)))                               \
-        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_MULT>), dgrid, dblock, lds_dma, g_stream, g, e);    \
-      break;                                                                                                \
-    default:                                                                                                \
-      if ((ok = raise_lds_limit<dw3x3_dma_kernel<S, PL, EPI_RAW>>(lds_dma)))                                \
-        hipLaunchKernelGGL((dw3x3_dma_kernel<S, PL, EPI_RAW>), dgrid, dblock, lds_dma, g_stream, g, e);     \
-      break;                                                                                                \
-  }
-      if (pl == 1) { DWD_MODE(2, 1) }
-      else { DWD_MODE(2, 0) }
-#undef DWD_MODE
-      if (ok) {
-        check_launch(fn);
-        return;
-      }
-      g.CSD = (g.NR * g.LWD) | 1;
-    }
 #define DW3L_MODE(S, PL, FULL)                                                                                        \
   switch (mode) {                                                                                                     \
     case EPI_BN: hipLaunchKernelGGL((dw3x3_lin_kernel<S, PL, EPI_BN, FULL>), grid, block, ldsl, g_stream, g, e); break;     \

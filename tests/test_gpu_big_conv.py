@@ -51,8 +51,8 @@ def test_big_conv(geom, flags, bn_bits):
     assert np.array_equal(got2[1], want[0])
 
 
-# ---- stride-2 depthwise layers large enough for the persistent kernel (bands staged by LDS-direct loads) ----
-# That kernel needs whole 64-channel groups, W % 4 == 0, Wo % 4 == 0 and at least two tiles per compute unit.
+# ---- stride-2 depthwise on whole 64-channel groups (bands staged by LDS-direct loads), at config-2 scale ----
+# That staging needs whole 64-channel groups, W % 4 == 0 and Wo % 4 == 0.
 DW_GEOMS = [
     # B, CH, H, W, pads (t, b, l, r)
     (130, 128, 56, 56, (1, 1, 1, 1)),    # config 2 geometry: four bands, the top one with a row above the image
