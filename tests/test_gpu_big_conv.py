@@ -103,6 +103,10 @@ DW1_GEOMS = [
     (4, 192, 45, 24, (0, 1, 0, 2)),      # no top / left padding, two bands, three channel groups
     (3, 64, 9, 112, (1, 1, 1, 1)),       # wide rows: the 64 KiB band limit applies instead of the 40 KiB one
     (2, 64, 6, 8, (1, 1, 1, 1)),         # a band shorter than one load instruction covers
+    # batches of several hundred images (more workgroups than the GPU holds at once)
+    (260, 128, 20, 20, (1, 1, 1, 1)),
+    (600, 64, 13, 56, (1, 1, 1, 1)),     # 14 column groups on 8 waves
+    (514, 64, 31, 40, (1, 0, 1, 1)),     # no bottom padding: 30 output rows
 ]
 
 
@@ -124,7 +128,14 @@ def test_depthwise_stride1_whole_groups(geom, flags, bn_bits):
     if not (relu and bn):
         shift = 19 if relu == 1 else 9
     got = depthwise_generic(x, wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
-    want = oracle.depthwise_generic(x, wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
-    assert got.shape == want.shape
-    assert np.array_equal(got, want), "depthwise mismatch"
+    sample = list(range(B)) if B <= 8 else sorted({0, 1, B // 2, B - 1})
+    want = oracle.depthwise_generic(x[sample], wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
+    assert got.shape[1:] == want.shape[1:]
+    assert np.array_equal(got[sample], want), "depthwise mismatch"
     assert want.max() > 0 and (want < 255).any(), "degenerate case"
+    if B > 8:
+        # a digest over many images against the same layer computed in small batches
+        step = 4
+        parts = [depthwise_generic(x[i:i + step], wt, b, k, lam, mult, shift, pads, (1, 1), relu, bn, bn_bits)
+                 for i in range(0, 24, step)]
+        assert np.array_equal(np.concatenate(parts), got[:24])
