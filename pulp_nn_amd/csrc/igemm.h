@@ -357,7 +357,7 @@ void igemm_kernel(ConvGeom g, EpiArgs e)
       R.amask = R.wmask = ~0u;
       // advance to the next K slice (scalar).  The prefetch runs one slice past the end; that
       // request repeats the last real slice instead, so no address beyond the caller's buffers is
-      // ever formed (buffer loads do not range-check the scalar offset).
+      // ever formed.
       if (u_slice + 1 < KT) {
         u_slice++;
         u_ci += IGEMM_BK;
