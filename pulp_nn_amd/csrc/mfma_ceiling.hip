@@ -12,6 +12,10 @@
 //      fragments and 32 MFMAs per wave, with and without a workgroup barrier per slice and with the
 //      fragment reads issued one slice ahead.  That is the main loop of igemm_dma_kernel with its
 //      global loads taken out: the rate it reaches bounds what that kernel structure can reach.
+//   3. The issue rate of the vector ALU for the instructions the depthwise kernels are made of (v_dot4,
+//      24-bit multiply-add, byte permute / align, DPP move, xor), at 1, 2 and 4 waves per SIMD, from the
+//      duration of a kernel of independent instruction chains: cycles per wave64 instruction per SIMD.
+//      With a kernel's SQ_INSTS_VALU count this gives the time its vector work alone needs.
 //
 // Build: hipcc --offload-arch=gfx950 -O3 -std=c++17 mfma_ceiling.hip -o ../lib/mfma_ceiling
 // (python -m pulp_nn_amd.build does it).  Run without arguments.
@@ -139,7 +143,64 @@ __global__ __launch_bounds__(512) void feed_kernel(int *out, long long *clk, int
   }
 }
 
+// ---- 3. vector ALU issue rate ---------------------------------------------------------------------------
+template <int OP>
+__global__ __launch_bounds__(1024) void valu_kernel(int *out, long long *clk, int iters)
+{
+  int a[8], b = threadIdx.x * 77 + 1, c = threadIdx.x ^ 0x1234567;
+  for (int i = 0; i < 8; i++) a[i] = threadIdx.x + i;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        if (OP == 0) asm volatile("v_dot4c_i32_i8 %0, %1, %2" : "+v"(a[i]) : "v"(b), "v"(c));
+        if (OP == 1) asm volatile("v_dot4_i32_i8 %0, %1, %2, %0" : "+v"(a[i]) : "v"(b), "v"(c));
+        if (OP == 2) asm volatile("v_mad_i32_i24 %0, %1, %2, %0" : "+v"(a[i]) : "v"(b), "v"(c));
+        if (OP == 3) asm volatile("v_perm_b32 %0, %1, %2, %0" : "+v"(a[i]) : "v"(b), "v"(c));
+        if (OP == 4) asm volatile("v_alignbyte_b32 %0, %1, %0, 3" : "+v"(a[i]) : "v"(b));
+        if (OP == 5) asm volatile("v_mov_b32_dpp %0, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(a[i]) : "v"(b));
+        if (OP == 6) asm volatile("v_xor_b32 %0, %1, %0" : "+v"(a[i]) : "v"(b));
+      }
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+  for (int i = 0; i < 8; i++) s += a[i];
+  out[blockIdx.x * 1024 + threadIdx.x] = s;
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    clk[0] = c1 - c0;
+    clk[1] = w1 - w0;
+  }
+}
+
 static int g_cus = 256;
+
+template <int OP>
+int run_valu(const char *name, int *out, long long *clk)
+{
+  const int iters = 20000;
+  hipEvent_t e0, e1;
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+  printf("%-18s", name);
+  for (int w = 1; w <= 4; w *= 2) {
+    hipLaunchKernelGGL(valu_kernel<OP>, dim3(g_cus), dim3(256 * w), 0, 0, out, clk, iters);
+    CK(hipEventRecord(e0, 0));
+    hipLaunchKernelGGL(valu_kernel<OP>, dim3(g_cus), dim3(256 * w), 0, 0, out, clk, iters);
+    CK(hipEventRecord(e1, 0));
+    CK(hipDeviceSynchronize());
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    long long h[2];
+    CK(hipMemcpy(h, clk, 16, hipMemcpyDeviceToHost));
+    const double mhz = (double)h[0] / (h[1] / 100.0);
+    printf("  %d waves/SIMD: %.2f cycles/instr/SIMD (%4.0f MHz)", w, ms * 1e-3 * mhz * 1e6 / (iters * 32.0 * w), mhz);
+  }
+  printf("\n");
+  fflush(stdout);
+  return 0;
+}
 
 template <typename K>
 int run(const char *name, K kern, int waves, long long mfma_per_wave_iter, int iters, int *out, long long *clk)
@@ -192,5 +253,13 @@ int main()
   run("reads, then MFMAs; barrier per slice", feed_kernel<0, 1>, 8, 32, 2000, out, clk);
   run("reads one slice ahead; no barrier", feed_kernel<1, 0>, 8, 32, 2000, out, clk);
   run("reads one slice ahead; barrier per slice", feed_kernel<1, 1>, 8, 32, 2000, out, clk);
+  printf("-- vector ALU: cycles per wave64 instruction per SIMD (one workgroup per compute unit, independent chains) --\n");
+  run_valu<0>("v_dot4c_i32_i8", out, clk);
+  run_valu<1>("v_dot4_i32_i8", out, clk);
+  run_valu<2>("v_mad_i32_i24", out, clk);
+  run_valu<3>("v_perm_b32", out, clk);
+  run_valu<4>("v_alignbyte_b32", out, clk);
+  run_valu<5>("v_mov_b32_dpp", out, clk);
+  run_valu<6>("v_xor_b32", out, clk);
   return 0;
 }
