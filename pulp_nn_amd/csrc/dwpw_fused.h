@@ -16,10 +16,12 @@
 // of four neighbouring pixels each and transposes it in registers into four pixels per channel; the
 // 3x3 windows are v_dot4 on byte windows; the requantised bytes are transposed back to four channels
 // of one pixel per lane and written to LDS.
-// Stage 2 (pointwise): 64 pixel x 64 channel blocks per wave, the weight fragments of a block fetched
-// straight from global memory in MFMA operand layout (all K slices of up to 256 bytes of K at once,
-// requested before stage 1 so that they arrive while it runs); 128 * sum_k w comes from one more MFMA
-// per fragment against a matrix of ones.
+// Stage 2 (pointwise): blocks of 16*TMB pixels x 64 channels, dealt to the waves; the weight fragments of a
+// block are fetched straight from global memory in MFMA operand layout, KP slices of K per pass (the first pass
+// of a wave's first block is requested before stage 1, so that it arrives while stage 1 runs; a wave's next
+// blocks of the same channel group reuse the fragments when one pass covers all of K); 128 * sum_k w comes from
+// one more MFMA per fragment against a matrix of ones; the per-channel constants of both layers are cached in
+// LDS; both epilogues pick their requantisation branch at run time.
 #pragma once
 #include "depthwise.h"
 #include "igemm.h"

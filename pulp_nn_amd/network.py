@@ -208,9 +208,11 @@ class Runner:
         L, N = self.layers[i], self.layers[i + 1]
         if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
             return False
-        # "auto": only where the single launch is not slower than the two (measured on MI355X at batch 256:
-        # planes up to 16 pixels wide; wider planes keep more of the machine busy as two launches)
-        if self.fuse_blocks == "auto" and self.shapes[L["in"]][1] > 16:
+        # "auto": only where the single launch is not slower than the two.  Measured on MI355X at batch 256
+        # (kernel times of the MobileNet chain's blocks): 16-pixel planes at stride 2 (11.2 us against 5.9 + 6.4) and
+        # 8-pixel planes at stride 1 (11.8 against 5.4 + 7.1) gain; 16-pixel planes at stride 1 (17.8 against
+        # 7.9 + 8.2), 8-pixel planes at stride 2, 4-pixel planes and everything wider lose.
+        if self.fuse_blocks == "auto" and (self.shapes[L["in"]][1], L["strides"][0]) not in ((16, 2), (8, 1)):
             return False
         if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
             return False
