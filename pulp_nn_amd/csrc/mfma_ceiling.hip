@@ -236,7 +236,8 @@ int main()
   CK(hipGetDevice(&dev));
   CK(hipGetDeviceProperties(&prop, dev));
   g_cus = prop.multiProcessorCount;
-  printf("%s, %d compute units; published dense int8 peak 5.0 POP/s = 16 cycles per 16x16x64 MFMA per SIMD at 2.4 GHz\n", prop.name, g_cus);
+  printf("%s (%s), %d compute units; published dense int8 peak 5.0 POP/s = 16 cycles per 16x16x64 MFMA per SIMD at 2.4 GHz\n",
+         prop.name[0] ? prop.name : "GPU", prop.gcnArchName, g_cus);
   int *out;
   long long *clk;
   CK(hipMalloc(&out, 4096 * 1024 * 4));
