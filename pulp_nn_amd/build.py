@@ -55,12 +55,33 @@ def build_tool(verbose=False):
     return tool_path()
 
 
+def demo_path():
+    return os.path.join(LIBDIR, "capi_demo")
+
+
+def build_demo(verbose=False):
+    """The plain C caller (csrc/capi_demo.c), compiled by gcc as C99 against include/ and linked with the 32-bit
+    library: what a reference-side application's build does.  Needs libpulpnn_hip32.so to exist."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c99", "-O2", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(os.path.dirname(HERE), "include"),
+           "-I", os.path.join(rocm, "include"), os.path.join(CSRC, "capi_demo.c"), "-o", demo_path(),
+           "-L", LIBDIR, "-lpulpnn_hip32", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("gcc failed:\n" + res.stdout)
+    return demo_path()
+
+
 def build_all(verbose=False):
     from concurrent.futures import ThreadPoolExecutor
     with ThreadPoolExecutor(3) as ex:
         libs = [ex.submit(build, b, verbose) for b in (32, 64)]
         tool = ex.submit(build_tool, verbose)
-        return [f.result() for f in libs] + [tool.result()]
+        out = [f.result() for f in libs] + [tool.result()]
+    return out + [build_demo(verbose)]
 
 
 if __name__ == "__main__":

@@ -56,7 +56,6 @@ static inline int pw_lds_bytes(int tn, int ks, int np, bool bn, int nw, int tm)
 template <int TN, int KS, int NP, int MODE, bool WIDE, int TM, int NW>
 __global__ __launch_bounds__(64 * NW, NW >= 8 ? 1 : 2) void pw_stream_kernel(PwGeom g, EpiArgs e)
 {
-  constexpr int BS = 64 * NW;      // threads per workgroup
   constexpr int PX = 16 * TM;      // pixels per step
   constexpr int CG = 16 * TN;      // channels per group
   constexpr int N = NP * CG;       // output channels
