@@ -101,6 +101,41 @@ def test_random_depthwise(case, bn_bits):
             assert_same(got2, want, "depthwise_hwc %s" % (case,))
 
 
+def _dw_group_cases(n, seed):
+    """Whole 64-channel groups with rows of whole dwords and output columns in whole groups of four: the shapes whose
+    bands are staged by LDS-direct loads (16-byte pieces that may straddle the image's first and last row)."""
+    r = rng_for(seed)
+    cases = []
+    while len(cases) < n:
+        ch = int(r.choice([64, 128, 192]))
+        w = 4 * int(r.integers(2, 16))
+        h = int(r.integers(3, 41))
+        s = int(r.integers(1, 3))
+        pads = (int(r.integers(0, 2)), int(r.integers(0, 2))) + [(1, 1), (1, 0), (0, 0)][int(r.integers(0, 3))]
+        ho, wo = (h + pads[0] + pads[1] - 3) // s + 1, (w + pads[2] + pads[3] - 3) // s + 1
+        if ho < 1 or wo < 1 or wo % 4:
+            continue
+        cases.append((int(r.choice([1, 2, 5])), ch, h, w, pads, s))
+    return cases
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("case", _dw_group_cases(40, 9102), ids=lambda c: "x".join(map(str, c[:4])) + "p%d%d%d%ds%d" % (c[4] + (c[5],)))
+def test_random_depthwise_whole_groups(case, bn_bits):
+    B, CH, H, W, pads, s = case
+    r = rng_for(hash(case) % (2 ** 31) + bn_bits)
+    relu, bn = _flags(r)
+    x, wt, b = rand_u8(r, (B, CH, H, W)), rand_s8(r, (CH, 3, 3)), rand_s8(r, (CH,))
+    if bn_bits == 32:
+        k, lam, bshift = r.integers(2 ** 12, 2 ** 14 + 1, CH), r.integers(-2 ** 16, 2 ** 16 + 1, CH), 16
+    else:
+        k, lam, bshift = r.integers(2 ** 20, 2 ** 24 + 1, CH), r.integers(-2 ** 36, 2 ** 36 + 1, CH), 28
+    shift = bshift if (relu and bn) else (14 if relu else 6)
+    want = oracle.depthwise_generic(x, wt, b, k, lam, 900, shift, pads, (s, s), relu, bn, bn_bits)
+    got = depthwise_generic(x, wt, b, k, lam, 900, shift, pads, (s, s), relu, bn, bn_bits)
+    assert_same(got, want, "depthwise %s" % (case,))
+
+
 def _linear_cases(n, seed):
     r = rng_for(seed)
     return [(int(r.choice([1, 2, 7, 64, 65, 130, 256, 257, 300])), int(r.choice([16, 32, 48, 100, 256, 1000, 37])),
