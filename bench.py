@@ -343,6 +343,47 @@ def main():
                        "images_per_s": round(256 / (wall * 1e-3), 1),
                        "mfma_frac": round(net["ops"] / (dev * 1e-3) / PEAK_INT8_OPS, 4),
                        "parity": "bit-exact (logits digest)" if ok else "MISMATCH"})
+        # one block of that chain on its own: 3x3 depthwise + pointwise on 8 x 8 x 256 planes, as one launch
+        # (pulp_nn_hip_dw_pw_hwc) and as the two launches the reference's call sequence makes
+        Lb = libs[32]
+        Lb.set_batch(256)
+        rb = np.random.Generator(np.random.PCG64(77))
+        Cb, Wb = 256, 8
+        xb = rb.integers(0, 256, (256, Wb, Wb, Cb), dtype=np.uint8)
+        dww = rb.integers(-128, 128, (Cb, 3, 3), dtype=np.int8)
+        pww = rb.integers(-128, 128, (Cb, Cb), dtype=np.int8)
+        kb1, lb1 = rb.integers(2 ** 12, 2 ** 14, Cb).astype(np.int32), rb.integers(-2 ** 16, 2 ** 16, Cb).astype(np.int32)
+        kb2, lb2 = rb.integers(2 ** 8, 2 ** 10, Cb).astype(np.int32), rb.integers(-2 ** 16, 2 ** 16, Cb).astype(np.int32)
+        sh1, sh2 = 16, 20
+        xbd, dwwd, pwwd = t(xb), t(dww), t(pww)
+        kb1d, lb1d, kb2d, lb2d = t(kb1), t(lb1), t(kb2), t(lb2)
+        mid = torch.zeros((256, Wb, Wb, Cb), dtype=torch.uint8, device="cuda")
+        ob1, ob2 = torch.zeros_like(mid), torch.zeros_like(mid)
+
+        def step_block_fused(i):
+            Lb.dw_pw_hwc(xbd, ob1, Wb, Wb, Cb, Wb, Wb, Cb, 1, dwwd, None, kb1d, lb1d, 0, sh1, 1, 1,
+                         pwwd, None, kb2d, lb2d, 0, sh2, 1, 1)
+
+        def step_block_two(i):
+            Lb.depthwise_hwc(xbd, None, mid, dwwd, kb1d, lb1d, 0, sh1, Wb, Wb, Cb, Wb, Wb, 1, 1, 1)
+            Lb.pulp_nn_pointwise_HoWo_parallel(mid, None, None, ob2, pwwd, kb2d, lb2d, 0, sh2, Wb, Wb, Cb, Wb, Wb, Cb,
+                                               1, 1, 0, 0, 0, 0, 1, 1, 1, 1)
+
+        _, dev_f, _ = time_launches(step_block_fused, steps, 5)
+        _, dev_t, _ = time_launches(step_block_two, steps, 5)
+        Lb.sync()
+        nchk = 8
+        want_mid = oracle.depthwise_generic(np.ascontiguousarray(xb[:nchk].transpose(0, 3, 1, 2)), dww, None, kb1, lb1, 0, sh1,
+                                            (1, 1, 1, 1), (1, 1), 1, 1)
+        want_b = oracle.pointwise(want_mid, pww, None, kb2, lb2, 0, sh2, 1, 1)
+        ok = np.array_equal(ob1[:nchk].cpu().numpy(), want_b) and np.array_equal(ob2.cpu().numpy(), ob1.cpu().numpy())
+        if not ok:
+            failures.append("cfg3 block")
+        blk_bytes = 2 * 256 * Wb * Wb * Cb + Cb * 9 + Cb * Cb + 4 * Cb * 4
+        layers.append({"layer": "cfg3_block_dw3x3_pw_8x8x256_b256", "ms": round(dev_f, 5), "ms_two_launches": round(dev_t, 5),
+                       "hbm_gbs": round(blk_bytes / (dev_f * 1e-3) / 1e9, 1), "hbm_frac": round(blk_bytes / (dev_f * 1e-3) / PEAK_HBM, 4),
+                       "parity": "bit-exact (8 images vs the oracle's two-layer chain; all images vs the two launches)" if ok else "MISMATCH",
+                       "note": "8.4 MB per launch: bound by launch and memory latency"})
         rec["layers"] = layers
 
     # ---- CPU baseline: the oracle on this machine's host cores --------------------
