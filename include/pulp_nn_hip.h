@@ -95,6 +95,33 @@ void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, un
                            void *pw_k, void *pw_lambda, unsigned short pw_out_mult, unsigned short pw_out_shift,
                            signed char pw_flag_relu, signed char pw_flag_batch_norm);
 
+/* The parameters of one such block, as pulp_nn_hip_dw_pw_hwc takes them. */
+typedef struct pulp_nn_hip_block {
+  const signed char *dw_wt, *dw_bias;
+  void *dw_k, *dw_lambda;
+  unsigned short dw_out_mult, dw_out_shift;
+  signed char dw_flag_relu, dw_flag_batch_norm;
+  const signed char *pw_weight, *pw_bias;
+  void *pw_k, *pw_lambda;
+  unsigned short pw_out_mult, pw_out_shift;
+  signed char pw_flag_relu, pw_flag_batch_norm;
+} pulp_nn_hip_block;
+
+/* n_blocks (1 to 8) such blocks of the same shape one after the other in one launch: stride 1, ch
+ * channels in and out of every layer, dim_im_x x dim_im_y pixels throughout (the run of identical
+ * blocks in the middle of a MobileNet).  No counterpart in the reference, which makes 2 x n_blocks
+ * calls with every intermediate tensor in memory.  Here a workgroup keeps its images' activations
+ * in LDS from block to block; only the last block's output is written.  blocks is a host array.
+ * The result is bit for bit that of n_blocks calls of pulp_nn_hip_dw_pw_hwc.  Supported: what
+ * pulp_nn_hip_dw_pw_hwc supports at stride 1 with ch_out == ch, images small enough for a
+ * workgroup to hold whole ones (dim_im_x x dim_im_y x ch x 2 bytes and the constants within 64 KB
+ * of LDS: 8 x 8 x 256, 16 x 16 x 64, 4 x 4 x 1024 ...), and a batch that is a multiple of the
+ * images a workgroup takes.  Anything else sets PULP_NN_HIP_ERR_UNSUPPORTED and queues nothing:
+ * call pulp_nn_hip_dw_pw_hwc per block instead. */
+void pulp_nn_hip_dw_pw_chain_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_x,
+                                 unsigned short dim_im_y, unsigned short ch, unsigned n_blocks,
+                                 const pulp_nn_hip_block *blocks);
+
 /* ---- calibration of out_shift -------------------------------------------------------
  * A network that requantises with batch-norm + ReLU chooses, per layer,
  * out_shift = floor(log2(max |acc * k[c]|)) - 7, the maximum taken over the batch, all

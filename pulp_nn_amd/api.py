@@ -7,6 +7,15 @@ from .build import lib_path
 _U16, _I8, _INT, _PTR = C.c_uint16, C.c_int8, C.c_int, C.c_void_p
 
 _CONV_ARGS = [_PTR] * 7 + [_U16] * 16 + [_INT, _INT]
+
+
+class HipBlock(C.Structure):
+    """pulp_nn_hip_block of include/pulp_nn_hip.h: the parameters of one depthwise + pointwise block."""
+    _fields_ = [("dw_wt", _PTR), ("dw_bias", _PTR), ("dw_k", _PTR), ("dw_lambda", _PTR),
+                ("dw_out_mult", _U16), ("dw_out_shift", _U16), ("dw_flag_relu", _I8), ("dw_flag_batch_norm", _I8),
+                ("pw_weight", _PTR), ("pw_bias", _PTR), ("pw_k", _PTR), ("pw_lambda", _PTR),
+                ("pw_out_mult", _U16), ("pw_out_shift", _U16), ("pw_flag_relu", _I8), ("pw_flag_batch_norm", _I8)]
+
 _DW_ARGS = [_PTR] * 8 + [_U16] * 16 + [_I8, _I8]
 
 CONV_NAMES = ("pulp_nn_conv_Ho_parallel", "pulp_nn_conv_Co_parallel", "pulp_nn_conv_HoWo_parallel",
@@ -87,6 +96,8 @@ class PulpNN:
         L.pulp_nn_hip_dw_pw_hwc.argtypes = ([_PTR] * 2 + [_U16] * 7 + [_PTR] * 4 + [_U16] * 2 + [_I8] * 2 + [_PTR] * 4 +
                                             [_U16] * 2 + [_I8] * 2)
         L.pulp_nn_hip_dw_pw_hwc.restype = None
+        L.pulp_nn_hip_dw_pw_chain_hwc.argtypes = [_PTR] * 2 + [_U16] * 3 + [C.c_uint, C.POINTER(HipBlock)]
+        L.pulp_nn_hip_dw_pw_chain_hwc.restype = None
         _U64 = C.c_uint64
         L.pulp_nn_hip_calib_workspace_bytes.argtypes, L.pulp_nn_hip_calib_workspace_bytes.restype = [_U64], _U64
         L.pulp_nn_hip_calib_conv.argtypes = [_PTR] * 4 + [_U16] * 12 + [_PTR, _U64, _PTR]
@@ -155,6 +166,19 @@ class PulpNN:
         self._call("pulp_nn_hip_dw_pw_hwc", _ptr(x), _ptr(out), dim_in_x, dim_in_y, ch, dim_out_x, dim_out_y, ch_out, stride,
                    _ptr(dw_wt), _ptr(dw_bias), _ptr(dw_k), _ptr(dw_lam), dw_mult, dw_shift, dw_relu, dw_bn,
                    _ptr(pw_w), _ptr(pw_bias), _ptr(pw_k), _ptr(pw_lam), pw_mult, pw_shift, pw_relu, pw_bn)
+
+    def dw_pw_chain_hwc(self, x, out, dim_x, dim_y, ch, blocks):
+        """Several depthwise + pointwise blocks of one shape (stride 1, ch channels throughout) in one launch.
+        blocks: a list of tuples (dw_wt, dw_bias, dw_k, dw_lam, dw_mult, dw_shift, dw_relu, dw_bn, pw_w, pw_bias,
+        pw_k, pw_lam, pw_mult, pw_shift, pw_relu, pw_bn), the arguments dw_pw_hwc takes per block.  Raises PulpNNError
+        (unsupported) where the blocks cannot be chained."""
+        arr = (HipBlock * len(blocks))()
+        for dst, b in zip(arr, blocks):
+            (dst.dw_wt, dst.dw_bias, dst.dw_k, dst.dw_lambda) = [_ptr(v) for v in b[0:4]]
+            (dst.dw_out_mult, dst.dw_out_shift, dst.dw_flag_relu, dst.dw_flag_batch_norm) = b[4:8]
+            (dst.pw_weight, dst.pw_bias, dst.pw_k, dst.pw_lambda) = [_ptr(v) for v in b[8:12]]
+            (dst.pw_out_mult, dst.pw_out_shift, dst.pw_flag_relu, dst.pw_flag_batch_norm) = b[12:16]
+        self._call("pulp_nn_hip_dw_pw_chain_hwc", _ptr(x), _ptr(out), dim_x, dim_y, ch, len(blocks), arr)
 
     # -- calibration ---------------------------------------------------------
     def calib_workspace_bytes(self, n_outputs):

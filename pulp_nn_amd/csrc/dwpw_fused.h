@@ -26,20 +26,31 @@
 #include "depthwise.h"
 #include "igemm.h"
 
-struct DwPwGeom {
-  const uint8_t *in;      // HWC [B][H][W][C]
+#define DWPW_MAX_BLOCKS 8  // blocks of one launch (pulp_nn_hip_dw_pw_chain_hwc)
+
+// one depthwise + pointwise block
+struct DwPwBlock {
   const int8_t *dw_wt;    // [C][3][3]
   const int8_t *dw_bias;  // int8 [C] or null
   const int8_t *pw_w;     // [Co][C]
   const int8_t *pw_bias;  // int8 [Co] or null
+  EpiArgs e_dw, e_pw;     // k, lambda, multiplier, shift of either layer
+  int mode_dw, mode_pw;   // requantisation branch of either layer (EPI_BN, EPI_MULT, EPI_RAW)
+};
+
+struct DwPwGeom {
+  const uint8_t *in;      // HWC [B][H][W][C]
   uint8_t *out;           // HWC [B][Ho][Wo][Co]
   int B, C, H, Ho, Co;
   int M;                  // B * Ho * Wo output pixels
   int BM;                 // pixels per tile: a multiple of 64 and of the pixels of a stage-1 item
   int KT;                 // 64-byte K slices: ceil(C / 64)
   int nsplit;             // workgroups that share a pixel tile, each computing Co / 64 / nsplit channel blocks
-  int mode_dw, mode_pw;   // requantisation branch of either layer (EPI_BN, EPI_MULT, EPI_RAW)
   FastDiv d_howo;         // division by Ho * Wo
+  // More than one block (stride 1, C == Co, tiles of whole images, nsplit == 1): block j + 1 reads the output of
+  // block j from LDS, where block j's epilogue left it in HWC order; only the last block writes to memory.
+  int nblocks;
+  DwPwBlock blk[DWPW_MAX_BLOCKS];
 };
 
 // LDS bytes of the activation operand: 64-byte K slices; with 16 or 32 channels a pixel's row is just its
@@ -53,7 +64,7 @@ __host__ __device__ static inline int dwpw_const_bytes(int nch) { return nch * (
 // is 16*TMB pixels x 64 channels.  KP: K slices whose weight fragments a wave holds at once (a pass over K).
 // The requantisation branches of both layers are run-time switches: one kernel per geometry, not nine.
 template <int WB, int R, int S, int NWV, int TMB, int KP>
-__global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g, EpiArgs e_dw, EpiArgs e_pw)
+__global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
 {
   constexpr int DWPW_WAVES = NWV;
   constexpr int BP = 16 * TMB;          // pixels of a stage-2 block
@@ -74,18 +85,23 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g, EpiArg
   const int HoWo = g.Ho * WO;
   const bool narrow = g.C < 64;                 // rows of C bytes instead of 64-byte K slices
 
-  // ---- stage 2 set-up: this wave's first block, its weight fragments requested now ----------------------
   const int MB = g.BM / BP;                     // pixel blocks of the tile
   const int NBT = (g.Co + 63) / 64;             // channel blocks of the layer
   const int nb_per = (NBT + g.nsplit - 1) / g.nsplit;
   const int nb_lo = part * nb_per, nb_hi = min(NBT, nb_lo + nb_per);
   const int nblk = MB * max(nb_hi - nb_lo, 0);  // blocks of this workgroup, dealt to the waves in turn
-  const __amdgpu_buffer_rsrc_t rsrc_w =
-      __builtin_amdgcn_make_buffer_rsrc((void *)g.pw_w, 0, (unsigned)g.Co * (unsigned)g.C, 0x00020000);
+  const int nch = max(nb_hi - nb_lo, 0) * 64;
+  int *c_bias = (int *)(dwpw_lds + dwpw_lds_bytes(g.BM, g.C));
+  bn_t *c_k = (bn_t *)(c_bias + nch), *c_l = c_k + nch;
+  // the output of a block that another block follows: [tile pixel][Co] bytes, the next block's HWC input
+  unsigned char *ylds = dwpw_lds + dwpw_lds_bytes(g.BM, g.C) + dwpw_const_bytes(nch);
   typedef unsigned v4u __attribute__((ext_vector_type(4)));
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+
   // weight fragment t of channel block nb: row i of the fragment is channel nb*64 + (i/4)*16 + 4*t + i%4, so that a
   // lane ends up with 16 consecutive channels (the order igemm.h uses)
-  auto load_w = [&](v4i (&wf)[KP][4], int nb, int kt0) {
+  auto load_w = [&](const int8_t *pw_w, v4i (&wf)[KP][4], int nb, int kt0) {
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)pw_w, 0, (unsigned)g.Co * (unsigned)g.C, 0x00020000);
 #pragma unroll
     for (int kk = 0; kk < KP; kk++)
 #pragma unroll
@@ -99,195 +115,233 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g, EpiArg
   };
   v4i wf[KP][4];
   int wf_nb = -1;  // channel block whose first-pass fragments wf holds
-  if (wave < nblk) {
-    wf_nb = nb_lo + wave / MB;
-    load_w(wf, wf_nb, 0);
-  }
-  // the pointwise layer's per-channel constants of this workgroup's channel blocks -> LDS (behind the activation
-  // operand), read by every block's epilogue
-  const int nch = max(nb_hi - nb_lo, 0) * 64;
-  int *c_bias = (int *)(dwpw_lds + dwpw_lds_bytes(g.BM, g.C));
-  bn_t *c_k = (bn_t *)(c_bias + nch), *c_l = c_k + nch;
-  for (int c = tid; c < nch; c += 64 * DWPW_WAVES) {
-    const int n = nb_lo * 64 + c;
-    const bool ok = n < g.Co;
-    c_bias[c] = (g.pw_bias && ok) ? (int)g.pw_bias[n] : 0;
-    c_k[c] = (g.mode_pw == EPI_BN && ok) ? e_pw.k[n] : (bn_t)0;
-    c_l[c] = (g.mode_pw == EPI_BN && ok) ? e_pw.lambda[n] : (bn_t)0;
-  }
+#pragma unroll 1
+  for (int j = 0; j < g.nblocks; j++) {
+    const DwPwBlock &P = g.blk[j];
+    const bool first = j == 0, last = j == g.nblocks - 1;
 
-  // ---- stage 1: depthwise into LDS ---------------------------------------------------------------------
-  {
-    const int CGN = g.C >= 64 ? g.C / 64 : 1;  // channel groups
-    const int LG = g.C >= 64 ? 1 : 64 / g.C;   // row groups inside a wave (fewer than 64 channels)
-    const int item_px = R * LG * WO;
-    const int nitems = (g.BM / item_px) * CGN;
-    const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
-    for (int it = wave; it < nitems; it += DWPW_WAVES) {
-      const int cg = it % CGN, seg = it / CGN;
-      const int lg = g.C >= 64 ? 0 : lane / g.C;
-      const int ch = g.C >= 64 ? cg * 64 + lane : lane % g.C;
-      const int mi = m0 + seg * item_px;  // first pixel of the item (all of it in one image)
-      if (mi >= g.M) break;
-      const int b = (int)fastdiv((unsigned)mi, g.d_howo);
-      const int oy0 = (mi - b * HoWo) / WO + lg * R;  // first output row of this lane's group
-      unsigned row[NIN][RD];
-      const uint8_t *src = g.in + ((long long)b * g.H * WB + (lane & 3)) * g.C + (ch & ~3);
+    // ---- stage 2 set-up ------------------------------------------------------------------------------------
+    // The pointwise layer's per-channel constants of this workgroup's channel blocks go to LDS (behind the
+    // activation operand), where every stage-2 block's epilogue reads them.  Their loads are issued first and the
+    // weight fragments' behind them: loads complete in order, so the wait for the constants leaves the fragments
+    // in flight.
+    constexpr int NCI = (1024 + 64 * DWPW_WAVES - 1) / (64 * DWPW_WAVES);  // at most 1024 output channels
+    int cb_[NCI];
+    bn_t ck_[NCI], cl_[NCI];
 #pragma unroll
-      for (int r = 0; r < NIN; r++) {
-        const int iy = oy0 * S - 1 + r;
-        const bool ok = (unsigned)iy < (unsigned)g.H;
-        const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB * g.C;
+    for (int q = 0; q < NCI; q++) {
+      const int c = tid + q * 64 * DWPW_WAVES, n = nb_lo * 64 + c;
+      const bool ok = c < nch && n < g.Co;
+      cb_[q] = (P.pw_bias && ok) ? (int)P.pw_bias[n] : 0;
+      ck_[q] = (P.mode_pw == EPI_BN && ok) ? P.e_pw.k[n] : (bn_t)0;
+      cl_[q] = (P.mode_pw == EPI_BN && ok) ? P.e_pw.lambda[n] : (bn_t)0;
+    }
+    // this wave's first stage-2 block: its weight fragments are requested now (first block of the launch; for the
+    // others the request went out behind the MFMAs of the block before)
+    if (first && wave < nblk) {
+      wf_nb = nb_lo + wave / MB;
+      load_w(P.pw_w, wf, wf_nb, 0);
+    }
 #pragma unroll
-        for (int d = 0; d < RD; d++) {
-          const unsigned v = *(const unsigned *)(rp + (long long)(4 * d) * g.C);
-          row[r][d] = ok ? v : 0u;
+    for (int q = 0; q < NCI; q++) {
+      const int c = tid + q * 64 * DWPW_WAVES;
+      if (c < nch) {
+        c_bias[c] = cb_[q];
+        c_k[c] = ck_[q];
+        c_l[c] = cl_[q];
+      }
+    }
+
+    // ---- stage 1: depthwise into LDS ---------------------------------------------------------------------
+    {
+      const int CGN = g.C >= 64 ? g.C / 64 : 1;  // channel groups
+      const int LG = g.C >= 64 ? 1 : 64 / g.C;   // row groups inside a wave (fewer than 64 channels)
+      const int item_px = R * LG * WO;
+      const int nitems = (g.BM / item_px) * CGN;
+      const unsigned sel1 = quad_sel1(lane), sel2 = quad_sel2(lane);
+      for (int it = wave; it < nitems; it += DWPW_WAVES) {
+        const int cg = it % CGN, seg = it / CGN;
+        const int lg = g.C >= 64 ? 0 : lane / g.C;
+        const int ch = g.C >= 64 ? cg * 64 + lane : lane % g.C;
+        const int mi = m0 + seg * item_px;  // first pixel of the item (all of it in one image)
+        if (mi >= g.M) break;
+        const int b = (int)fastdiv((unsigned)mi, g.d_howo);
+        const int oy0 = (mi - b * HoWo) / WO + lg * R;  // first output row of this lane's group
+        unsigned row[NIN][RD];
+        // the image this item lies in: in memory for the first block, else where the block before left it (a tile of
+        // several blocks is made of whole images, stride 1: image (b - first image of the tile) of the tile)
+        const uint8_t *img = first ? g.in + (long long)b * g.H * WB * g.C
+                                   : ylds + (long long)(b - (int)fastdiv((unsigned)m0, g.d_howo)) * g.H * WB * g.C;
+        const uint8_t *src = img + (lane & 3) * g.C + (ch & ~3);
+#pragma unroll
+        for (int r = 0; r < NIN; r++) {
+          const int iy = oy0 * S - 1 + r;
+          const bool ok = (unsigned)iy < (unsigned)g.H;
+          const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB * g.C;
+#pragma unroll
+          for (int d = 0; d < RD; d++) {
+            const unsigned v = *(const unsigned *)(rp + (long long)(4 * d) * g.C);
+            row[r][d] = ok ? v : 0u;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < NIN; r++)
+#pragma unroll
+          for (int d = 0; d < RD; d++) row[r][d] = quad_transpose4x4_perm(row[r][d], sel1, sel2) ^ 0x80808080u;
+        unsigned wA[3], wB[3];
+        int wsum = 0;
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+          const int8_t *p = P.dw_wt + (long long)ch * 9 + 3 * i;
+          const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
+          wA[i] = k0 | (k1 << 8) | (k2 << 16);
+          wB[i] = wA[i] << 8;
+          wsum += (int)p[0] + (int)p[1] + (int)p[2];
+        }
+        const int corr = 128 * wsum + (P.dw_bias ? (int)P.dw_bias[ch] : 0);
+        bn_t kk = 0, ll = 0;
+        if (P.mode_dw == EPI_BN) {
+          kk = P.e_dw.k[ch];
+          ll = P.e_dw.lambda[ch];
+        }
+        const int dw_mult = P.e_dw.mult, dw_shift = P.e_dw.shift;
+        const bool fastq = (P.mode_dw == EPI_BN) ? __all(bn_k_small(kk)) : (dw_shift >= 16);
+        // after the quad transpose this lane holds channels (ch & ~3) .. + 3 of pixel column 4*xg + lane%4:
+        // one dword of the activation operand, K slice (ch / 64), 16-byte chunk (ch % 64) / 16
+        const int c4 = ch & ~3;
+        unsigned char *abase = narrow ? dwpw_lds + c4 : dwpw_lds + (c4 >> 6) * (g.BM * 64) + (c4 & 15);
+        const int chunk = (c4 & 63) >> 4;
+        const int pl0 = seg * item_px + lg * R * WO + (lane & 3);  // tile-local pixel of row 0, column lane % 4
+        auto body = [&](auto md, auto fq) {
+          constexpr int MODE_DW = decltype(md)::value;
+          constexpr bool FASTQ = decltype(fq)::value;
+#pragma unroll
+          for (int ro = 0; ro < R; ro++) {
+#pragma unroll
+            for (int xg = 0; xg < XG; xg++) {
+              int acc[4] = {corr, corr, corr, corr};
+#pragma unroll
+              for (int i = 0; i < 3; i++) {
+                unsigned span[NS];
+#pragma unroll
+                for (int d = 0; d < NS; d++) {
+                  const int col = xg * S - 1 + d;  // dword column
+                  span[d] = (col >= 0 && col < RD) ? row[ro * S + i][col < 0 ? 0 : (col >= RD ? RD - 1 : col)] : 0x80808080u;
+                }
+                dw_tap<O0, NS>(span, wA[i], wB[i], acc[0]);
+                dw_tap<O0 + S, NS>(span, wA[i], wB[i], acc[1]);
+                dw_tap<O0 + 2 * S, NS>(span, wA[i], wB[i], acc[2]);
+                dw_tap<O0 + 3 * S, NS>(span, wA[i], wB[i], acc[3]);
+              }
+              unsigned packed = requant4_same<MODE_DW, FASTQ>(acc[0], acc[1], acc[2], acc[3], kk, ll, dw_mult, dw_shift);
+              packed = quad_transpose4x4_perm(packed, sel1, sel2) ^ 0x80808080u;
+              const int pl = pl0 + ro * WO + 4 * xg;
+              *(unsigned *)(abase + (narrow ? pl * g.C : pl * 64 + ((chunk ^ ((pl >> 1) & 3)) << 4))) = packed;
+            }
+          }
+        };
+        if (P.mode_dw == EPI_BN) {
+          if (fastq) body(std::integral_constant<int, EPI_BN>{}, std::true_type{});
+          else body(std::integral_constant<int, EPI_BN>{}, std::false_type{});
+        } else if (P.mode_dw == EPI_MULT) {
+          if (fastq) body(std::integral_constant<int, EPI_MULT>{}, std::true_type{});
+          else body(std::integral_constant<int, EPI_MULT>{}, std::false_type{});
+        } else {
+          body(std::integral_constant<int, EPI_RAW>{}, std::false_type{});
         }
       }
+    }
+    __syncthreads();
+
+    // ---- stage 2: pointwise from LDS ---------------------------------------------------------------------
+    const int swz = (lgrp ^ ((l16 >> 1) & 3)) << 4;
+    // narrow rows: chunk lgrp of a row if it exists, else chunk 0 (multiplied by zero weights)
+    const int nar_off = l16 * g.C + ((16 * lgrp < g.C) ? 16 * lgrp : 0);
+    const int pw_mult = P.e_pw.mult, pw_shift = P.e_pw.shift;
+    for (int blk = wave; blk < nblk; blk += DWPW_WAVES) {
+      const int mb = blk % MB, nb = nb_lo + blk / MB;
+      v4i acc[4][TMB], wacc[4];
 #pragma unroll
-      for (int r = 0; r < NIN; r++)
+      for (int t = 0; t < 4; t++) {
+        wacc[t] = (v4i){0, 0, 0, 0};
 #pragma unroll
-        for (int d = 0; d < RD; d++) row[r][d] = quad_transpose4x4_perm(row[r][d], sel1, sel2) ^ 0x80808080u;
-      unsigned wA[3], wB[3];
-      int wsum = 0;
-#pragma unroll
-      for (int i = 0; i < 3; i++) {
-        const int8_t *p = g.dw_wt + (long long)ch * 9 + 3 * i;
-        const unsigned k0 = (uint8_t)p[0], k1 = (uint8_t)p[1], k2 = (uint8_t)p[2];
-        wA[i] = k0 | (k1 << 8) | (k2 << 16);
-        wB[i] = wA[i] << 8;
-        wsum += (int)p[0] + (int)p[1] + (int)p[2];
+        for (int s = 0; s < TMB; s++) acc[t][s] = (v4i){0, 0, 0, 0};
       }
-      const int corr = 128 * wsum + (g.dw_bias ? (int)g.dw_bias[ch] : 0);
-      bn_t kk = 0, ll = 0;
-      if (g.mode_dw == EPI_BN) {
-        kk = e_dw.k[ch];
-        ll = e_dw.lambda[ch];
-      }
-      const bool fastq = (g.mode_dw == EPI_BN) ? __all(bn_k_small(kk)) : (e_dw.shift >= 16);
-      // after the quad transpose this lane holds channels (ch & ~3) .. + 3 of pixel column 4*xg + lane%4:
-      // one dword of the activation operand, K slice (ch / 64), 16-byte chunk (ch % 64) / 16
-      const int c4 = ch & ~3;
-      unsigned char *abase = narrow ? dwpw_lds + c4 : dwpw_lds + (c4 >> 6) * (g.BM * 64) + (c4 & 15);
-      const int chunk = (c4 & 63) >> 4;
-      const int pl0 = seg * item_px + lg * R * WO + (lane & 3);  // tile-local pixel of row 0, column lane % 4
-      auto body = [&](auto md, auto fq) {
-        constexpr int MODE_DW = decltype(md)::value;
-        constexpr bool FASTQ = decltype(fq)::value;
+      for (int kt0 = 0; kt0 < g.KT; kt0 += KP) {
+        // (the first pass of the first block was requested before stage 1; a wave's next blocks of the same channel
+        // block re-use the fragments when one pass covers K)
+        if (kt0 > 0 || wf_nb != nb || g.KT > KP) {
+          load_w(P.pw_w, wf, nb, kt0);
+          wf_nb = kt0 == 0 ? nb : -1;
+        }
 #pragma unroll
-        for (int ro = 0; ro < R; ro++) {
+        for (int kk = 0; kk < KP; kk++) {
+          if (kt0 + kk < g.KT) {
+            const unsigned char *ab = narrow ? dwpw_lds + mb * BP * g.C + nar_off
+                                             : dwpw_lds + (kt0 + kk) * (g.BM * 64) + (mb * BP + l16) * 64 + swz;
+            const int sstep = narrow ? 16 * g.C : 1024;  // 16 rows on
+            v4i af[TMB];
 #pragma unroll
-          for (int xg = 0; xg < XG; xg++) {
-            int acc[4] = {corr, corr, corr, corr};
+            for (int s = 0; s < TMB; s++) af[s] = *(const v4i *)(ab + s * sstep);
 #pragma unroll
-            for (int i = 0; i < 3; i++) {
-              unsigned span[NS];
+            for (int t = 0; t < 4; t++) {
 #pragma unroll
-              for (int d = 0; d < NS; d++) {
-                const int col = xg * S - 1 + d;  // dword column
-                span[d] = (col >= 0 && col < RD) ? row[ro * S + i][col < 0 ? 0 : (col >= RD ? RD - 1 : col)] : 0x80808080u;
-              }
-              dw_tap<O0, NS>(span, wA[i], wB[i], acc[0]);
-              dw_tap<O0 + S, NS>(span, wA[i], wB[i], acc[1]);
-              dw_tap<O0 + 2 * S, NS>(span, wA[i], wB[i], acc[2]);
-              dw_tap<O0 + 3 * S, NS>(span, wA[i], wB[i], acc[3]);
+              for (int s = 0; s < TMB; s++) acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[kk][t], af[s], acc[t][s], 0, 0, 0);
+              wacc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[kk][t], ones, wacc[t], 0, 0, 0);
             }
-            unsigned packed = requant4_same<MODE_DW, FASTQ>(acc[0], acc[1], acc[2], acc[3], kk, ll, e_dw.mult, e_dw.shift);
-            packed = quad_transpose4x4_perm(packed, sel1, sel2) ^ 0x80808080u;
-            const int pl = pl0 + ro * WO + 4 * xg;
-            *(unsigned *)(abase + (narrow ? pl * g.C : pl * 64 + ((chunk ^ ((pl >> 1) & 3)) << 4))) = packed;
+          }
+        }
+      }
+      // the last stage-2 block of this wave in this block of the chain: the weight fragments of its first one in the
+      // next block are requested now, so that they travel while the epilogue, the barrier and the next depthwise
+      // stage run
+      if (!last && blk + DWPW_WAVES >= nblk) {
+        wf_nb = nb_lo + wave / MB;
+        load_w(g.blk[j + 1].pw_w, wf, wf_nb, 0);
+      }
+      // epilogue: acc[t][s][r] = channel cb + 4*t + r of pixel m0 + mb*BP + 16*s + l16; wacc[t][r] = sum of that channel's weights
+      const int cb = nb * 64 + lgrp * 16;
+      const bool acc24 = g.C <= 256;  // |acc| <= K * 255 * 128 + 128 < 2^23
+      unsigned packed[TMB][4];
+      auto requantise = [&](auto md) {
+        constexpr int MODE_PW = decltype(md)::value;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          int corr[4];
+          bn_t kk[4], ll[4];
+          bool ks = true;
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int c = cb + 4 * t + r - nb_lo * 64;  // channel inside this workgroup's range (constants past Co are zero)
+            kk[r] = (MODE_PW == EPI_BN) ? c_k[c] : (bn_t)0;
+            ll[r] = (MODE_PW == EPI_BN) ? c_l[c] : (bn_t)0;
+            ks = ks && bn_k_small(kk[r]);
+            corr[r] = c_bias[c] + 128 * wacc[t][r];
+          }
+          const bool k_small = __all(ks);
+#pragma unroll
+          for (int s = 0; s < TMB; s++) {
+            const int a0 = acc[t][s][0] + corr[0], a1 = acc[t][s][1] + corr[1];
+            const int a2 = acc[t][s][2] + corr[2], a3 = acc[t][s][3] + corr[3];
+            packed[s][t] = acc24 ? requant4<MODE_PW, true>(a0, a1, a2, a3, kk, ll, k_small, pw_mult, pw_shift)
+                                 : requant4<MODE_PW, false>(a0, a1, a2, a3, kk, ll, k_small, pw_mult, pw_shift);
           }
         }
       };
-      if (g.mode_dw == EPI_BN) {
-        if (fastq) body(std::integral_constant<int, EPI_BN>{}, std::true_type{});
-        else body(std::integral_constant<int, EPI_BN>{}, std::false_type{});
-      } else if (g.mode_dw == EPI_MULT) {
-        if (fastq) body(std::integral_constant<int, EPI_MULT>{}, std::true_type{});
-        else body(std::integral_constant<int, EPI_MULT>{}, std::false_type{});
-      } else {
-        body(std::integral_constant<int, EPI_RAW>{}, std::false_type{});
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- stage 2: pointwise from LDS ---------------------------------------------------------------------
-  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const int swz = (lgrp ^ ((l16 >> 1) & 3)) << 4;
-  // narrow rows: chunk lgrp of a row if it exists, else chunk 0 (multiplied by zero weights)
-  const int nar_off = l16 * g.C + ((16 * lgrp < g.C) ? 16 * lgrp : 0);
-  for (int blk = wave; blk < nblk; blk += DWPW_WAVES) {
-    const int mb = blk % MB, nb = nb_lo + blk / MB;
-    v4i acc[4][TMB], wacc[4];
+      if (P.mode_pw == EPI_BN) requantise(std::integral_constant<int, EPI_BN>{});
+      else if (P.mode_pw == EPI_MULT) requantise(std::integral_constant<int, EPI_MULT>{});
+      else requantise(std::integral_constant<int, EPI_RAW>{});
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      wacc[t] = (v4i){0, 0, 0, 0};
-#pragma unroll
-      for (int s = 0; s < TMB; s++) acc[t][s] = (v4i){0, 0, 0, 0};
-    }
-    for (int kt0 = 0; kt0 < g.KT; kt0 += KP) {
-      // (the first pass of the first block was requested before stage 1; a wave's next blocks of the same channel
-      // block re-use the fragments when one pass covers K)
-      if (kt0 > 0 || wf_nb != nb || g.KT > KP) {
-        load_w(wf, nb, kt0);
-        wf_nb = kt0 == 0 ? nb : -1;
-      }
-#pragma unroll
-      for (int kk = 0; kk < KP; kk++) {
-        if (kt0 + kk < g.KT) {
-          const unsigned char *ab = narrow ? dwpw_lds + mb * BP * g.C + nar_off
-                                           : dwpw_lds + (kt0 + kk) * (g.BM * 64) + (mb * BP + l16) * 64 + swz;
-          const int sstep = narrow ? 16 * g.C : 1024;  // 16 rows on
-          v4i af[TMB];
-#pragma unroll
-          for (int s = 0; s < TMB; s++) af[s] = *(const v4i *)(ab + s * sstep);
-#pragma unroll
-          for (int t = 0; t < 4; t++) {
-#pragma unroll
-            for (int s = 0; s < TMB; s++) acc[t][s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[kk][t], af[s], acc[t][s], 0, 0, 0);
-            wacc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[kk][t], ones, wacc[t], 0, 0, 0);
-          }
+      for (int s = 0; s < TMB; s++) {
+        const int pl = mb * BP + 16 * s + l16;  // tile-local pixel
+        if (m0 + pl < g.M && cb < g.Co) {
+          const v4i v = {(int)packed[s][0], (int)packed[s][1], (int)packed[s][2], (int)packed[s][3]};
+          if (last) *(v4i *)(g.out + (long long)(m0 + pl) * g.Co + cb) = v;
+          else *(v4i *)(ylds + pl * g.Co + cb) = v;
         }
       }
     }
-    // epilogue: acc[t][s][r] = channel cb + 4*t + r of pixel m0 + mb*BP + 16*s + l16; wacc[t][r] = sum of that channel's weights
-    const int cb = nb * 64 + lgrp * 16;
-    const bool acc24 = g.C <= 256;  // |acc| <= K * 255 * 128 + 128 < 2^23
-    unsigned packed[TMB][4];
-    auto requantise = [&](auto md) {
-      constexpr int MODE_PW = decltype(md)::value;
-#pragma unroll
-      for (int t = 0; t < 4; t++) {
-        int corr[4];
-        bn_t kk[4], ll[4];
-        bool ks = true;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int c = cb + 4 * t + r - nb_lo * 64;  // channel inside this workgroup's range (constants past Co are zero)
-          kk[r] = (MODE_PW == EPI_BN) ? c_k[c] : (bn_t)0;
-          ll[r] = (MODE_PW == EPI_BN) ? c_l[c] : (bn_t)0;
-          ks = ks && bn_k_small(kk[r]);
-          corr[r] = c_bias[c] + 128 * wacc[t][r];
-        }
-        const bool k_small = __all(ks);
-#pragma unroll
-        for (int s = 0; s < TMB; s++) {
-          const int a0 = acc[t][s][0] + corr[0], a1 = acc[t][s][1] + corr[1];
-          const int a2 = acc[t][s][2] + corr[2], a3 = acc[t][s][3] + corr[3];
-          packed[s][t] = acc24 ? requant4<MODE_PW, true>(a0, a1, a2, a3, kk, ll, k_small, e_pw.mult, e_pw.shift)
-                               : requant4<MODE_PW, false>(a0, a1, a2, a3, kk, ll, k_small, e_pw.mult, e_pw.shift);
-        }
-      }
-    };
-    if (g.mode_pw == EPI_BN) requantise(std::integral_constant<int, EPI_BN>{});
-    else if (g.mode_pw == EPI_MULT) requantise(std::integral_constant<int, EPI_MULT>{});
-    else requantise(std::integral_constant<int, EPI_RAW>{});
-#pragma unroll
-    for (int s = 0; s < TMB; s++) {
-      const int m = m0 + mb * BP + 16 * s + l16;
-      if (m < g.M && cb < g.Co)
-        *(v4i *)(g.out + (long long)m * g.Co + cb) = (v4i){(int)packed[s][0], (int)packed[s][1], (int)packed[s][2], (int)packed[s][3]};
-    }
+    // the next block reads this one's output and rewrites the activation operand and the constants
+    if (!last) __syncthreads();
   }
 }

@@ -1035,28 +1035,33 @@ void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bi
                    epi_mode(flag_relu, flag_batch_norm, true), true);
 }
 
-void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_in_x,
-                           unsigned short dim_im_in_y, unsigned short ch, unsigned short dim_im_out_x,
-                           unsigned short dim_im_out_y, unsigned short ch_out, unsigned short stride,
-                           const signed char *dw_wt, const signed char *dw_bias, void *dw_k, void *dw_lambda,
-                           unsigned short dw_out_mult, unsigned short dw_out_shift, signed char dw_flag_relu,
-                           signed char dw_flag_batch_norm, const signed char *pw_weight, const signed char *pw_bias,
-                           void *pw_k, void *pw_lambda, unsigned short pw_out_mult, unsigned short pw_out_shift,
-                           signed char pw_flag_relu, signed char pw_flag_batch_norm)
+// Common part of pulp_nn_hip_dw_pw_hwc (one block) and pulp_nn_hip_dw_pw_chain_hwc (several).
+static void dwpw_common(const char *fn, const unsigned char *Im_in, unsigned char *Im_out, int W, int H, int C, int Wo_arg,
+                        int Ho_arg, int Co, int S, unsigned n_blocks, const pulp_nn_hip_block *blocks)
 {
-  const char *fn = __func__;
-  REQUIRE(Im_in && Im_out && dw_wt && pw_weight, PULP_NN_HIP_ERR_ARGUMENT, "null activation or weight pointer");
-  REQUIRE(dim_im_in_x && dim_im_in_y && ch && ch_out && (stride == 1 || stride == 2), PULP_NN_HIP_ERR_ARGUMENT,
-          "zero dimension or stride other than 1 or 2");
-  const int W = dim_im_in_x, H = dim_im_in_y, C = ch, Co = ch_out, S = stride;
+  REQUIRE(Im_in && Im_out && blocks && n_blocks >= 1, PULP_NN_HIP_ERR_ARGUMENT, "null activation pointer or no block");
+  REQUIRE(n_blocks <= DWPW_MAX_BLOCKS, PULP_NN_HIP_ERR_ARGUMENT, "too many blocks for one launch");
+  REQUIRE(W && H && C && Co && (S == 1 || S == 2), PULP_NN_HIP_ERR_ARGUMENT, "zero dimension or stride other than 1 or 2");
   const int Wo = (W - 1) / S + 1, Ho = (H - 1) / S + 1;
-  REQUIRE(dim_im_out_x == Wo && dim_im_out_y == Ho, PULP_NN_HIP_ERR_ARGUMENT, "output size is not that of a 3x3 window with padding 1");
-  const int mode_dw = epi_mode(dw_flag_relu, dw_flag_batch_norm, true);  // pulp_nn_depthwise_generic.c:167-178 tests FLAG_RELU for truth
-  const int mode_pw = epi_mode(pw_flag_relu, pw_flag_batch_norm);
-  EpiArgs e_dw, e_pw;
-  REQUIRE(epi_args(mode_dw, (bn_t *)dw_k, (bn_t *)dw_lambda, dw_out_mult, dw_out_shift, &e_dw) &&
-              epi_args(mode_pw, (bn_t *)pw_k, (bn_t *)pw_lambda, pw_out_mult, pw_out_shift, &e_pw),
-          PULP_NN_HIP_ERR_ARGUMENT, "out_shift out of range or null k/lambda");
+  REQUIRE(Wo_arg == Wo && Ho_arg == Ho, PULP_NN_HIP_ERR_ARGUMENT, "output size is not that of a 3x3 window with padding 1");
+  DwPwGeom g;
+  g.nblocks = (int)n_blocks;
+  bool w_aligned = true;
+  for (unsigned j = 0; j < n_blocks; j++) {
+    const pulp_nn_hip_block &b = blocks[j];
+    REQUIRE(b.dw_wt && b.pw_weight, PULP_NN_HIP_ERR_ARGUMENT, "null weight pointer");
+    DwPwBlock &P = g.blk[j];
+    P.dw_wt = (const int8_t *)b.dw_wt;
+    P.dw_bias = (const int8_t *)b.dw_bias;
+    P.pw_w = (const int8_t *)b.pw_weight;
+    P.pw_bias = (const int8_t *)b.pw_bias;
+    P.mode_dw = epi_mode(b.dw_flag_relu, b.dw_flag_batch_norm, true);  // pulp_nn_depthwise_generic.c:167-178 tests FLAG_RELU for truth
+    P.mode_pw = epi_mode(b.pw_flag_relu, b.pw_flag_batch_norm);
+    REQUIRE(epi_args(P.mode_dw, (bn_t *)b.dw_k, (bn_t *)b.dw_lambda, b.dw_out_mult, b.dw_out_shift, &P.e_dw) &&
+                epi_args(P.mode_pw, (bn_t *)b.pw_k, (bn_t *)b.pw_lambda, b.pw_out_mult, b.pw_out_shift, &P.e_pw),
+            PULP_NN_HIP_ERR_ARGUMENT, "out_shift out of range or null k/lambda");
+    w_aligned = w_aligned && aligned(b.pw_weight, 16);
+  }
   // per input width and stride: output rows of a stage-1 item, waves per workgroup, pixels / 16 of a stage-2 block
   int R = 0, NWV = 4, TMB = 2;
   if (W == 64) R = 2;
@@ -1068,15 +1073,10 @@ void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, un
   const int LG = C >= 64 ? 1 : 64 / C, CGN = C >= 64 ? C / 64 : 1;
   const long long M = (long long)g_batch * Ho * Wo;
   const bool ok = R > 0 && c_ok && Ho % (R * LG) == 0 && Co % 16 == 0 && aligned(Im_in, 4) && aligned(Im_out, 16) &&
-                  aligned(pw_weight, 16) && M <= 0x7fffffffLL && (long long)Co * C < 0x7fffffffLL;
+                  w_aligned && M <= 0x7fffffffLL && (long long)Co * C < 0x7fffffffLL;
   if (!ok)
     return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "no fused kernel for this geometry: call the depthwise and the pointwise layer separately");
-  DwPwGeom g;
   g.in = Im_in;
-  g.dw_wt = (const int8_t *)dw_wt;
-  g.dw_bias = (const int8_t *)dw_bias;
-  g.pw_w = (const int8_t *)pw_weight;
-  g.pw_bias = (const int8_t *)pw_bias;
   g.out = Im_out;
   g.B = (int)g_batch;
   g.C = C;
@@ -1085,8 +1085,6 @@ void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, un
   g.Co = Co;
   g.M = (int)M;
   g.KT = (C + 63) / 64;
-  g.mode_dw = mode_dw;
-  g.mode_pw = mode_pw;
   g.d_howo = fastdiv_make((unsigned)(Ho * Wo));
   // a tile: enough stage-1 items (item_px pixels x 64 channels each) to give every wave one, in whole stage-2 blocks
   const int item_px = R * LG * Wo, bp = 16 * TMB;
@@ -1096,18 +1094,33 @@ void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, un
     segs--;
   while ((segs * item_px) % bp) segs++;
   g.BM = segs * item_px;
-  const int tiles = (int)((M + g.BM - 1) / g.BM), nbt = (Co + 63) / 64;
+  int tiles = (int)((M + g.BM - 1) / g.BM);
+  const int nbt = (Co + 63) / 64;
   // few pixel tiles: several workgroups share one, each with a part of the output channels (and its own copy of stage 1)
   g.nsplit = 1;
   while (tiles * g.nsplit < num_cus() && g.nsplit * 2 <= nbt) g.nsplit *= 2;
-  const size_t lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(((nbt + g.nsplit - 1) / g.nsplit) * 64);
+  size_t lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(((nbt + g.nsplit - 1) / g.nsplit) * 64);
+  if (n_blocks > 1) {
+    // Several blocks: the output of one is the next one's input and stays in LDS, so a tile has to be whole images
+    // (the 3x3 window of a pixel then never leaves the tile), the blocks have to keep the shape (stride 1, as many
+    // channels out as in), and a workgroup computes all channels.
+    const int img_px = Ho * Wo;
+    int per_tile = (g.BM + img_px - 1) / img_px;  // images per tile
+    while ((per_tile * img_px) % bp || (per_tile * img_px) % item_px) per_tile++;
+    g.BM = per_tile * img_px;
+    tiles = (int)((M + g.BM - 1) / g.BM);
+    g.nsplit = 1;
+    lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(nbt * 64) + (size_t)g.BM * Co;
+    if (S != 1 || C != Co || g_batch % (unsigned)per_tile != 0)
+      return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "blocks can only be chained at stride 1 with as many channels out as in, on whole images per tile");
+  }
   if (lds > 65536)
     return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "no fused kernel for this geometry: call the depthwise and the pointwise layer separately");
   const dim3 grid((unsigned)(tiles * g.nsplit)), block(64 * NWV);
-#define DWPW_KP(WB, RR, SS, NW, TM)                                                                                   \
-  if (g.KT == 1) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 1>), grid, block, lds, g_stream, g, e_dw, e_pw);      \
-  else if (g.KT == 2) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 2>), grid, block, lds, g_stream, g, e_dw, e_pw); \
-  else hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 4>), grid, block, lds, g_stream, g, e_dw, e_pw);
+#define DWPW_KP(WB, RR, SS, NW, TM)                                                                    \
+  if (g.KT == 1) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 1>), grid, block, lds, g_stream, g);      \
+  else if (g.KT == 2) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 2>), grid, block, lds, g_stream, g); \
+  else hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 4>), grid, block, lds, g_stream, g);
   if (W == 64 && S == 1) { DWPW_KP(64, 2, 1, 4, 2) }
   else if (W == 64) { DWPW_KP(64, 2, 2, 4, 2) }
   else if (W == 32 && S == 1) { DWPW_KP(32, 4, 1, 4, 2) }
@@ -1119,6 +1132,27 @@ void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, un
   else { DWPW_KP(4, 4, 1, 8, 2) }
 #undef DWPW_KP
   check_launch(fn);
+}
+
+void pulp_nn_hip_dw_pw_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_in_x,
+                           unsigned short dim_im_in_y, unsigned short ch, unsigned short dim_im_out_x,
+                           unsigned short dim_im_out_y, unsigned short ch_out, unsigned short stride,
+                           const signed char *dw_wt, const signed char *dw_bias, void *dw_k, void *dw_lambda,
+                           unsigned short dw_out_mult, unsigned short dw_out_shift, signed char dw_flag_relu,
+                           signed char dw_flag_batch_norm, const signed char *pw_weight, const signed char *pw_bias,
+                           void *pw_k, void *pw_lambda, unsigned short pw_out_mult, unsigned short pw_out_shift,
+                           signed char pw_flag_relu, signed char pw_flag_batch_norm)
+{
+  const pulp_nn_hip_block b = {dw_wt,     dw_bias,   dw_k,        dw_lambda,    dw_out_mult,  dw_out_shift, dw_flag_relu, dw_flag_batch_norm,
+                               pw_weight, pw_bias,   pw_k,        pw_lambda,    pw_out_mult,  pw_out_shift, pw_flag_relu, pw_flag_batch_norm};
+  dwpw_common(__func__, Im_in, Im_out, dim_im_in_x, dim_im_in_y, ch, dim_im_out_x, dim_im_out_y, ch_out, stride, 1, &b);
+}
+
+void pulp_nn_hip_dw_pw_chain_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_x,
+                                 unsigned short dim_im_y, unsigned short ch, unsigned n_blocks,
+                                 const pulp_nn_hip_block *blocks)
+{
+  dwpw_common(__func__, Im_in, Im_out, dim_im_x, dim_im_y, ch, dim_im_x, dim_im_y, ch, 1, n_blocks, blocks);
 }
 
 void pulp_nn_depthwise_3x3_s1(uint8_t *In_Img, uint8_t *Out_Img, int R, int C, int CH, int p_l, int p_r,

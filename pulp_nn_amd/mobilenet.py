@@ -103,11 +103,14 @@ class Runner(network.Runner):
     kernel for it; otherwise, and with fused=False, the chain is the reference's:
     pulp_nn_hip_hwc_to_chw + pulp_nn_depthwise_generic.  fuse_blocks: a depthwise layer and the
     pointwise layer behind it run as one launch (pulp_nn_hip_dw_pw_hwc); the depthwise results are
-    then not materialised (self.activations holds stale buffers for them)."""
+    then not materialised (self.activations holds stale buffers for them).  chain_blocks: the run of
+    five identical blocks on 8 x 8 x 256 is one launch (pulp_nn_hip_dw_pw_chain_hwc); only its last
+    output is materialised."""
 
-    def __init__(self, nn, net, fused=True, fuse_blocks="auto"):
+    def __init__(self, nn, net, fused=True, fuse_blocks="auto", chain_blocks=True):
         self.net = net
-        super().__init__(nn, descriptor(net), (128, 128, 3), net["batch"], fused=fused, fuse_blocks=fuse_blocks)
+        super().__init__(nn, descriptor(net), (128, 128, 3), net["batch"], fused=fused, fuse_blocks=fuse_blocks,
+                         chain_blocks=chain_blocks)
         self.logits = self.act["fc"].view(net["batch"], 1000)
         self.activations = [self.act[L["name"]] for L in net["layers"]]
 

@@ -80,11 +80,13 @@ def infer_shapes(layers, input_shape):
 class Runner:
     """Uploads the parameters once, owns the activation buffers and queues the chain."""
 
-    def __init__(self, nn, layers, input_shape, batch, fused=True, fuse_blocks="auto"):
+    def __init__(self, nn, layers, input_shape, batch, fused=True, fuse_blocks="auto", chain_blocks=True):
         import torch
         self.nn, self.layers, self.batch, self.torch = nn, layers, batch, torch
         self.fused, self.unfused = fused, set()
         self.fuse_blocks, self.unfused_blocks, self.launches = fuse_blocks, set(), 0
+        # runs of depthwise + pointwise blocks of one shape as one launch each (pulp_nn_hip_dw_pw_chain_hwc)
+        self.chain_blocks, self.unchained = bool(chain_blocks and fused and fuse_blocks), set()
         self.shapes = infer_shapes(layers, input_shape)
         bn_np = np.int64 if nn.bn_bits == 64 else np.int32
 
@@ -191,6 +193,12 @@ class Runner:
         i = 0
         while i < len(self.layers):
             L = self.layers[i]
+            n = self._chain_length(i) if self.chain_blocks else 0
+            if n >= 2 and self._queue_chain(i, n, tensors):
+                last = self.layers[i + 2 * n - 1]["name"]
+                out = tensors[last] = self.act[last]
+                i += 2 * n
+                continue
             if self._block_fusable(i) and self._queue_block(i, tensors):
                 out = tensors[self.layers[i + 1]["name"]] = self.act[self.layers[i + 1]["name"]]
                 i += 2
@@ -201,8 +209,9 @@ class Runner:
         return out
 
     # -- depthwise + pointwise as one launch ------------------------------------------------
-    def _block_fusable(self, i):
-        """Layer i is a 3x3 / padding 1 depthwise layer whose only reader is the pointwise layer i + 1."""
+    def _block_fusable(self, i, policy=True):
+        """Layer i is a 3x3 / padding 1 depthwise layer whose only reader is the pointwise layer i + 1.
+        policy=False: only whether the block can be one launch, not whether it pays on its own."""
         if not (self.fused and self.fuse_blocks) or i in self.unfused_blocks or i + 1 >= len(self.layers):
             return False
         L, N = self.layers[i], self.layers[i + 1]
@@ -212,7 +221,7 @@ class Runner:
         # (kernel times of the MobileNet chain's blocks): 16-pixel planes at stride 2 (11.2 us against 5.9 + 6.4) and
         # 8-pixel planes at stride 1 (11.8 against 5.4 + 7.1) gain; 16-pixel planes at stride 1 (17.8 against
         # 7.9 + 8.2), 8-pixel planes at stride 2, 4-pixel planes and everything wider lose.
-        if self.fuse_blocks == "auto" and (self.shapes[L["in"]][1], L["strides"][0]) not in ((16, 2), (8, 1)):
+        if policy and self.fuse_blocks == "auto" and (self.shapes[L["in"]][1], L["strides"][0]) not in ((16, 2), (8, 1)):
             return False
         if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
             return False
@@ -221,6 +230,46 @@ class Runner:
             return False
         readers = [M for M in self.layers if (M["in"] == L["name"] or (M["op"] == "add" and L["name"] in M["in"]))]
         return len(readers) == 1
+
+    def _readers(self, name):
+        return [M for M in self.layers if (M["in"] == name or (M["op"] == "add" and name in M["in"]))]
+
+    def _chain_length(self, i):
+        """How many depthwise + pointwise blocks of one shape start at layer i (stride 1, as many channels out as in,
+        every intermediate tensor read by the next layer only): such a run is one launch, with the activations kept
+        in LDS from block to block."""
+        if i in self.unchained:
+            return 0
+        n, shape = 0, None
+        while n < 8 and self._block_fusable(i + 2 * n, policy=False):
+            L, N = self.layers[i + 2 * n], self.layers[i + 2 * n + 1]
+            if L["strides"][0] != 1 or self.shapes[L["in"]] != self.shapes[N["name"]]:
+                break
+            if shape is None:
+                shape = self.shapes[L["in"]]
+            if self.shapes[L["in"]] != shape or (n > 0 and len(self._readers(L["in"])) != 1):
+                break
+            n += 1
+        return n
+
+    def _queue_chain(self, i, n, tensors):
+        nn = self.nn
+        H, W, Cc = self.shapes[self.layers[i]["in"]]
+        blocks = []
+        for j in range(n):
+            L, P, N, Q = self.layers[i + 2 * j], self.params[i + 2 * j], self.layers[i + 2 * j + 1], self.params[i + 2 * j + 1]
+            k1, l1, m1, s1, r1, b1 = self._requant_args(L, P)
+            k2, l2, m2, s2, r2, b2 = self._requant_args(N, Q)
+            blocks.append((P["w"], P.get("bias"), k1, l1, m1, s1, r1, b1, Q["w"], Q.get("bias"), k2, l2, m2, s2, r2, b2))
+        try:
+            nn.dw_pw_chain_hwc(tensors[self.layers[i]["in"]], self.act[self.layers[i + 2 * n - 1]["name"]], W, H, Cc, blocks)
+        except PulpNNError as err:
+            if err.code != 2:
+                raise
+            self.unchained.add(i)    # these blocks cannot share a launch
+            return False
+        self.launches += 1
+        return True
 
     def _queue_block(self, i, tensors):
         L, P, N, Q, nn = self.layers[i], self.params[i], self.layers[i + 1], self.params[i + 1], self.nn

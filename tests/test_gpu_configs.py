@@ -78,7 +78,7 @@ def test_config3_mobilenet_batch256():
     # two images through the oracle chain, every intermediate layer kept
     want_logits, want_layers = cfg3_oracle.forward(net, net["x"][:2], keep=True)
     # 1. every depthwise + pointwise block as one launch: 16 launches, the depthwise results never materialised
-    runner = mobilenet.Runner(L, net, fuse_blocks=True)
+    runner = mobilenet.Runner(L, net, fuse_blocks=True, chain_blocks=False)
     got = runner.run(x)
     L.sync()
     L.set_batch(1)
@@ -102,13 +102,22 @@ def test_config3_mobilenet_batch256():
     assert_same(got[:2], want_logits, "config 3 logits")
     check_digest("cfg3_b256_logits", got)
     assert not runner.unfused, "depthwise layers without a fused kernel: %s" % sorted(runner.unfused)
-    # 3. the runner's default: blocks fused where that is not slower (6 of the 13 here)
+    # 3. the runner's default: the five identical blocks on 8 x 8 x 256 as one launch, of the others those fused
+    # that are not slower that way (one here)
     auto = mobilenet.Runner(L, net)
     got3 = auto.run(x)
     L.sync()
     L.set_batch(1)
-    assert auto.launches == 23, auto.launches
+    assert auto.launches == 19, auto.launches
+    assert not auto.unchained
     check_digest("cfg3_b256_logits", got3.cpu().numpy())
+    # ... and with every block fused: 12 launches
+    allf = mobilenet.Runner(L, net, fuse_blocks=True)
+    got4 = allf.run(x)
+    L.sync()
+    L.set_batch(1)
+    assert allf.launches == 12, allf.launches
+    check_digest("cfg3_b256_logits", got4.cpu().numpy())
     # 4. the same chain with the layout changes as separate launches (the reference's call sequence)
     plain = mobilenet.Runner(L, net, fused=False)
     got2 = plain.run(x)

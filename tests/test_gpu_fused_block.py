@@ -104,3 +104,72 @@ def test_fused_block_rejects_what_it_cannot_do():
     assert err.value.code == 2
     with pytest.raises(PulpNNError):                                           # wrong output size
         L.dw_pw_hwc(x, out, 16, 16, 64, 15, 16, 64, 1, w9, None, None, None, 300, 15, 1, 0, pw, None, None, None, 300, 15, 1, 0)
+
+
+# ---- several blocks of one shape in one launch (pulp_nn_hip_dw_pw_chain_hwc) --------------------------------------
+# B, H, W, C, number of blocks.  Whole images per workgroup: 8 x 8 x 256 (one image), 4 x 4 x 512 (two images, so
+# an even batch), 16 x 16 x 64 (one image), 8 x 8 x 64 with 16-channel-multiple counts
+CHAINS = [
+    (7, 8, 8, 256, 5),       # the run of five identical blocks of the MobileNet chain
+    (6, 4, 4, 512, 3),
+    (5, 16, 16, 64, 2),
+    (4, 8, 8, 128, 8),       # the most blocks one launch takes
+    (9, 8, 8, 64, 1),        # a single block through the chain entry point
+]
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+@pytest.mark.parametrize("flags", [((1, 1), (1, 1)), ((1, 0), (1, 1)), ((1, 1), (1, 0))], ids=lambda f: "dw%d%d_pw%d%d" % (f[0] + f[1]))
+@pytest.mark.parametrize("geom", CHAINS, ids=lambda g: "x".join(map(str, g)))
+def test_block_chain(geom, flags, bn_bits):
+    B, H, W, C, nb = geom
+    r = rng_for(4711 + bn_bits + 5 * flags[0][1] + flags[1][1] + nb)
+    x = rand_u8(r, (B, H, W, C))
+    cur = x
+    blocks, keep = [], []
+    for j in range(nb):
+        dw = dict(w=rand_s8(r, (C, 3, 3)), bias=rand_s8(r, (C,)) if j % 2 == 0 else None, **layer_params(r, C, flags[0], bn_bits))
+        pw = dict(w=rand_s8(r, (C, 1, 1, C)), bias=rand_s8(r, (C,)) if j % 2 else None, **layer_params(r, C, flags[1], bn_bits))
+        # shifts from the layers' own accumulators (the oracle walks the chain), so that every layer produces real values
+        dw["shift"] = pick_shift(dw, int(9 ** 0.5 * 128 * 74 * 2))
+        mid = oracle.depthwise_generic(np.ascontiguousarray(cur.transpose(0, 3, 1, 2)), dw["w"], dw["bias"], dw["k"], dw["lam"],
+                                       dw["mult"], dw["shift"], (1, 1, 1, 1), (1, 1), dw["relu"], dw["bn"], bn_bits)
+        acc = mid.reshape(-1, C).astype(np.int64) @ pw["w"].reshape(C, C).astype(np.int64).T
+        pw["shift"] = pick_shift(pw, int(np.abs(acc).max()))
+        cur = oracle.pointwise(mid, pw["w"], pw["bias"], pw["k"], pw["lam"], pw["mult"], pw["shift"], pw["relu"], pw["bn"], bn_bits)
+        assert cur.max() > 0 and (cur < 255).any(), "degenerate block %d" % j
+        dev_args = (dev(dw["w"]), dev(dw["bias"]), bn_dev(dw["k"], bn_bits), bn_dev(dw["lam"], bn_bits), dw["mult"], dw["shift"],
+                    dw["relu"], dw["bn"], dev(pw["w"]), dev(pw["bias"]), bn_dev(pw["k"], bn_bits), bn_dev(pw["lam"], bn_bits),
+                    pw["mult"], pw["shift"], pw["relu"], pw["bn"])
+        keep.append(dev_args)
+        blocks.append(dev_args)
+    L = nn(bn_bits)
+    out = torch.full((B, H, W, C), 0xA5, dtype=torch.uint8, device="cuda")
+    L.set_batch(B)
+    try:
+        L.dw_pw_chain_hwc(dev(x), out, W, H, C, blocks)
+        L.sync()
+    finally:
+        L.set_batch(1)
+    assert np.array_equal(out.cpu().numpy(), cur), "chain of %d blocks differs from the oracle's 2 x %d layers" % (nb, nb)
+
+
+def test_block_chain_rejects_what_it_cannot_do():
+    L = nn(32)
+    z = lambda *s: torch.zeros(s, dtype=torch.int8, device="cuda")
+    blk = lambda C: (z(C, 9), None, None, None, 300, 15, 1, 0, z(C, C), None, None, None, 300, 15, 1, 0)
+    x = torch.zeros((3, 4, 4, 512), dtype=torch.uint8, device="cuda")
+    L.set_batch(3)                      # two 4 x 4 images per workgroup: an odd batch cannot be chained
+    try:
+        with pytest.raises(PulpNNError) as err:
+            L.dw_pw_chain_hwc(x, torch.zeros_like(x), 4, 4, 512, [blk(512)] * 2)
+        assert err.value.code == 2
+        x = torch.zeros((3, 32, 32, 64), dtype=torch.uint8, device="cuda")   # 32 x 32 x 64 x 2 bytes: too large for LDS
+        with pytest.raises(PulpNNError) as err:
+            L.dw_pw_chain_hwc(x, torch.zeros_like(x), 32, 32, 64, [blk(64)] * 2)
+        assert err.value.code == 2
+        with pytest.raises(PulpNNError) as err:                                 # more blocks than one launch takes
+            L.dw_pw_chain_hwc(x, torch.zeros_like(x), 32, 32, 64, [blk(64)] * 9)
+        assert err.value.code == 1
+    finally:
+        L.set_batch(1)
