@@ -22,6 +22,13 @@
 // blocks of the same channel group reuse the fragments when one pass covers all of K); 128 * sum_k w comes from
 // one more MFMA per fragment against a matrix of ones; the per-channel constants of both layers are cached in
 // LDS; both epilogues pick their requantisation branch at run time.
+//
+// Several blocks of one shape (stride 1, as many channels out as in) run back to back in one launch: a tile is
+// then made of whole images, so that the 3x3 window of a pixel never leaves it; the epilogue of a block writes
+// its bytes to LDS in HWC order instead of to memory, the depthwise stage of the next block reads them from
+// there, and only the last block's output leaves the chip.  The blocks' parameters are an array in the kernel
+// arguments.  The weight fragments of a wave's first stage-2 block of the next block are requested behind the
+// MFMAs of its last one in this block: they travel during the epilogue, the barrier and the next depthwise stage.
 #pragma once
 #include "depthwise.h"
 #include "igemm.h"
