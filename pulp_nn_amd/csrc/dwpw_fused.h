@@ -70,7 +70,8 @@ __host__ __device__ static inline int dwpw_const_bytes(int nch) { return nch * (
 // WB, R, S: input width, output rows per stage-1 item, stride.  NWV: waves per workgroup.  TMB: a stage-2 block
 // is 16*TMB pixels x 64 channels.  KP: K slices whose weight fragments a wave holds at once (a pass over K).
 // The requantisation branches of both layers are run-time switches: one kernel per geometry, not nine.
-template <int WB, int R, int S, int NWV, int TMB, int KP>
+// CHAIN: g.nblocks blocks back to back; otherwise the one block g.blk[0], with nothing of the chain's loop left.
+template <int WB, int R, int S, int NWV, int TMB, int KP, bool CHAIN = false>
 __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
 {
   constexpr int DWPW_WAVES = NWV;
@@ -122,10 +123,11 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
   };
   v4i wf[KP][4];
   int wf_nb = -1;  // channel block whose first-pass fragments wf holds
+  const int nblocks = CHAIN ? g.nblocks : 1;
 #pragma unroll 1
-  for (int j = 0; j < g.nblocks; j++) {
-    const DwPwBlock &P = g.blk[j];
-    const bool first = j == 0, last = j == g.nblocks - 1;
+  for (int j = 0; j < nblocks; j++) {
+    const DwPwBlock &P = g.blk[CHAIN ? j : 0];
+    const bool first = !CHAIN || j == 0, last = !CHAIN || j == nblocks - 1;
 
     // ---- stage 2 set-up ------------------------------------------------------------------------------------
     // The pointwise layer's per-channel constants of this workgroup's channel blocks go to LDS (behind the
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
       // stage run
       if (!last && blk + DWPW_WAVES >= nblk) {
         wf_nb = nb_lo + wave / MB;
-        load_w(g.blk[j + 1].pw_w, wf, wf_nb, 0);
+        load_w(g.blk[CHAIN ? j + 1 : 0].pw_w, wf, wf_nb, 0);
       }
       // epilogue: acc[t][s][r] = channel cb + 4*t + r of pixel m0 + mb*BP + 16*s + l16; wacc[t][r] = sum of that channel's weights
       const int cb = nb * 64 + lgrp * 16;

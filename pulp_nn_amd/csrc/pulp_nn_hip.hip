@@ -1121,6 +1121,20 @@ static void dwpw_common(const char *fn, const unsigned char *Im_in, unsigned cha
   if (g.KT == 1) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 1>), grid, block, lds, g_stream, g);      \
   else if (g.KT == 2) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 2>), grid, block, lds, g_stream, g); \
   else hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, SS, NW, TM, 4>), grid, block, lds, g_stream, g);
+#define DWPW_CHAIN_KP(WB, RR, NW, TM)                                                                                     \
+  if (g.KT == 1) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, 1, NW, TM, 1, true>), grid, block, lds, g_stream, g);      \
+  else if (g.KT == 2) hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, 1, NW, TM, 2, true>), grid, block, lds, g_stream, g); \
+  else hipLaunchKernelGGL((dwpw_fused_kernel<WB, RR, 1, NW, TM, 4, true>), grid, block, lds, g_stream, g);
+  if (n_blocks > 1) {
+    // (stride 1 only; the widest planes never fit the LDS of a chained launch)
+    if (W == 32) { DWPW_CHAIN_KP(32, 4, 4, 2) }
+    else if (W == 16) { DWPW_CHAIN_KP(16, 4, 8, 2) }
+    else if (W == 8) { DWPW_CHAIN_KP(8, 4, 8, 2) }
+    else if (W == 4) { DWPW_CHAIN_KP(4, 4, 8, 2) }
+    else return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "blocks of this width cannot be chained");
+    check_launch(fn);
+    return;
+  }
   if (W == 64 && S == 1) { DWPW_KP(64, 2, 1, 4, 2) }
   else if (W == 64) { DWPW_KP(64, 2, 2, 4, 2) }
   else if (W == 32 && S == 1) { DWPW_KP(32, 4, 1, 4, 2) }
@@ -1131,6 +1145,7 @@ static void dwpw_common(const char *fn, const unsigned char *Im_in, unsigned cha
   else if (W == 8) { DWPW_KP(8, 2, 2, 8, 2) }
   else { DWPW_KP(4, 4, 1, 8, 2) }
 #undef DWPW_KP
+#undef DWPW_CHAIN_KP
   check_launch(fn);
 }
 
