@@ -85,6 +85,8 @@ struct ConvGeom {
   int batch;           // number of images: ceil(M / HoWo)
   int ci_shift;        // log2(Ci) when Ci is a power of two (GATHER_SUBTAP), else 0
   int rkx;             // 65536 / kx + 1: t * rkx >> 16 == t / kx for t < 32 (GATHER_SUBTAP)
+  int cpt;             // Ci / 64: K sub-slices per filter tap (igemm_ring_kernel)
+  FastDiv d_cpt, d_kx; // divisions by cpt and kx (igemm_ring_kernel)
 };
 
 #define IGEMM_BK 64

@@ -23,6 +23,7 @@
 #include <stdio.h>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 #define CK(x)                                                              \
   do {                                                                     \
     hipError_t e_ = (x);                                                   \
@@ -71,6 +72,44 @@ __global__ __launch_bounds__(64 * W) void reg_kernel(int *out, long long *clk, i
   int s = 0;
   for (int i = 0; i < NA; i++)
     for (int j = 0; j < NB; j++) s += acc[i][j].x + acc[i][j].y + acc[i][j].z + acc[i][j].w;
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s + lds[threadIdx.x & 1];
+  if (threadIdx.x == 0) {
+    clk[2 * blockIdx.x] = c1 - c0;
+    clk[2 * blockIdx.x + 1] = w1 - w0;
+  }
+}
+
+
+// the same with v_mfma_i32_32x32x32_i8 (16 accumulator registers per MFMA, 65536 op, 32 cycles per SIMD at peak)
+template <int NA, int NB, int RND, int W>
+__global__ __launch_bounds__(64 * W) void reg32_kernel(int *out, long long *clk, int iters)
+{
+  extern __shared__ int lds[];
+  v4i a[NA], b[NB];
+  for (int q = 0; q < NA; q++) {
+    const unsigned s = threadIdx.x * 131 + q * 7919 + blockIdx.x;
+    a[q] = RND ? (v4i){(int)hash32(s), (int)hash32(s + 1), (int)hash32(s + 2), (int)hash32(s + 3)} : (v4i){(int)threadIdx.x & 3, 1, 2, 3};
+  }
+  for (int q = 0; q < NB; q++) {
+    const unsigned s = threadIdx.x * 137 + q * 7907 + blockIdx.x + 99;
+    b[q] = RND ? (v4i){(int)hash32(s), (int)hash32(s + 1), (int)hash32(s + 2), (int)hash32(s + 3)} : (v4i){5, (int)threadIdx.x & 3, 7, 8};
+  }
+  v16i acc[NA][NB];
+  for (int i = 0; i < NA; i++)
+    for (int j = 0; j < NB; j++)
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < NA; i++)
+#pragma unroll
+      for (int j = 0; j < NB; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+  for (int i = 0; i < NA; i++)
+    for (int j = 0; j < NB; j++)
+      for (int r = 0; r < 16; r++) s += acc[i][j][r];
   out[blockIdx.x * blockDim.x + threadIdx.x] = s + lds[threadIdx.x & 1];
   if (threadIdx.x == 0) {
     clk[2 * blockIdx.x] = c1 - c0;
@@ -143,6 +182,110 @@ __global__ __launch_bounds__(512) void feed_kernel(int *out, long long *clk, int
   }
 }
 
+
+// the same wave tile on v_mfma_i32_32x32x32_i8: a fragment is 32 rows x 32 bytes of K (lane l: row l%32,
+// 16-byte chunk l/32 of the K step), per 64-byte K slice again twelve ds_read_b128, 32 xor, and 16 MFMAs
+template <int PIPE, int BAR>
+__global__ __launch_bounds__(512) void feed32_kernel(int *out, long long *clk, int iters)
+{
+  extern __shared__ __attribute__((aligned(16))) unsigned char feed_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+  for (int i = tid; i < 65536 / 4; i += 512) ((unsigned *)feed_lds)[i] = hash32(i + blockIdx.x * 77);
+  __syncthreads();
+  // K step ks of row r: chunk 2*ks + lh in slot chunk ^ ((r/2)%4)
+  const int sw = (l32 >> 1) & 3;
+  const int o0 = ((0 + lh) ^ sw) << 4, o1 = ((2 + lh) ^ sw) << 4;
+  const unsigned char *a_lane = feed_lds + ((wave & 1) * 128 + l32) * 64;
+  const unsigned char *w_lane = feed_lds + 32768 + ((wave >> 1) * 64 + l32) * 64;
+  v16i acc[2][4];
+  for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++)
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+  struct Frags {
+    v4i wf[2][2], af[4][2];
+  };
+  volatile int slot_mask = 1;
+  auto read = [&](Frags &F, int j) {
+    const int slot = (j & slot_mask) * 16384;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      F.wf[t][0] = *(const v4i *)(w_lane + slot + t * 2048 + o0);
+      F.wf[t][1] = *(const v4i *)(w_lane + slot + t * 2048 + o1);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      F.af[s][0] = *(const v4i *)(a_lane + slot + s * 2048 + o0);
+      F.af[s][1] = *(const v4i *)(a_lane + slot + s * 2048 + o1);
+    }
+  };
+  auto multiply = [&](Frags &F) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        const v4i a = F.af[s][ks] ^ (int)0x80808080;
+#pragma unroll
+        for (int t = 0; t < 2; t++) acc[t][s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(F.wf[t][ks], a, acc[t][s], 0, 0, 0);
+      }
+  };
+  Frags F0, F1;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  if (PIPE == 0) {
+    for (int it = 0; it < iters; it++) {
+      if (BAR) __builtin_amdgcn_s_barrier();
+      read(F0, it);
+      multiply(F0);
+    }
+  } else {
+    read(F0, 0);
+    for (int it = 0; it < iters; it += 2) {
+      if (BAR) __builtin_amdgcn_s_barrier();
+      read(F1, it + 1);
+      multiply(F0);
+      if (BAR) __builtin_amdgcn_s_barrier();
+      read(F0, it + 2);
+      multiply(F1);
+    }
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  int s = 0;
+  for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 4; j++)
+      for (int r = 0; r < 16; r++) s += acc[i][j][r];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  if (threadIdx.x == 0) {
+    clk[2 * blockIdx.x] = c1 - c0;
+    clk[2 * blockIdx.x + 1] = w1 - w0;
+  }
+}
+
+// LDS read bandwidth: W waves per SIMD reading conflict-free 16-byte fragments back to back
+__global__ __launch_bounds__(1024) void ldsbw_kernel(int *out, long long *clk, int iters)
+{
+  extern __shared__ __attribute__((aligned(16))) unsigned char feed_lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, lgrp = lane >> 4;
+  for (int i = tid; i < 65536 / 4; i += blockDim.x) ((unsigned *)feed_lds)[i] = hash32(i);
+  __syncthreads();
+  const unsigned char *p = feed_lds + (((wave & 7) * 64 + l16) * 64) + ((lgrp ^ ((l16 >> 1) & 3)) << 4);
+  v4i acc = {0, 0, 0, 0};
+  volatile int slot_mask = 1;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; it++) {
+    const int slot = (it & slot_mask) * 32768;
+    v4i v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = *(const v4i *)(p + slot + (u & 3) * 1024);
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc ^= v[u];
+  }
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  out[blockIdx.x * blockDim.x + threadIdx.x] = acc.x + acc.y + acc.z + acc.w;
+  if (threadIdx.x == 0) {
+    clk[2 * blockIdx.x] = c1 - c0;
+    clk[2 * blockIdx.x + 1] = w1 - w0;
+  }
+}
+
 // ---- 3. vector ALU issue rate ---------------------------------------------------------------------------
 template <int OP>
 __global__ __launch_bounds__(1024) void valu_kernel(int *out, long long *clk, int iters)
@@ -203,7 +346,7 @@ int run_valu(const char *name, int *out, long long *clk)
 }
 
 template <typename K>
-int run(const char *name, K kern, int waves, long long mfma_per_wave_iter, int iters, int *out, long long *clk)
+int run(const char *name, K kern, int waves, long long mfma_per_wave_iter, int iters, int *out, long long *clk, int op_per_mfma = 32768)
 {
   hipEvent_t e0, e1;
   CK(hipEventCreate(&e0));
@@ -222,7 +365,7 @@ int run(const char *name, K kern, int waves, long long mfma_per_wave_iter, int i
   CK(hipMemcpy(h, clk, 16, hipMemcpyDeviceToHost));
   const double mfmas = (double)reps * g_cus * waves * iters * mfma_per_wave_iter;
   const double mhz = (double)h[0] / (h[1] / 100.0);
-  const double pops = mfmas * 32768 / (ms * 1e-3) / 1e15;
+  const double pops = mfmas * op_per_mfma / (ms * 1e-3) / 1e15;
   printf("%-58s %d waves/SIMD  %6.3f POP/s  %4.0f MHz  %5.1f cycles/MFMA/SIMD\n", name, waves / 4, pops, mhz,
          (ms * 1e-3) * mhz * 1e6 / (mfmas / (g_cus * 4.0)));
   fflush(stdout);
@@ -249,11 +392,41 @@ int main()
   run("random bytes, 16 accumulators", reg_kernel<4, 4, 1, 16>, 16, 16, 2500, out, clk);
   run("random bytes, 32 accumulators", reg_kernel<4, 8, 1, 8>, 8, 32, 1250, out, clk);
   run("random bytes, 32 accumulators", reg_kernel<4, 8, 1, 4>, 4, 32, 1250, out, clk);
+  printf("-- registers only, v_mfma_i32_32x32x32_i8 (cycles per MFMA: 32 at peak) --\n");
+  run("32x32x32, constant operands, 8 accumulators of 16", reg32_kernel<2, 4, 0, 8>, 8, 8, 2500, out, clk, 65536);
+  run("32x32x32, constant operands, 8 accumulators of 16", reg32_kernel<2, 4, 0, 4>, 4, 8, 2500, out, clk, 65536);
+  run("32x32x32, random bytes, 8 accumulators of 16", reg32_kernel<2, 4, 1, 8>, 8, 8, 2500, out, clk, 65536);
+  run("32x32x32, random bytes, 8 accumulators of 16", reg32_kernel<2, 4, 1, 4>, 4, 8, 2500, out, clk, 65536);
   printf("-- operands from LDS: 12 ds_read_b128 + 32 xor + 32 MFMA per wave and K slice, random bytes --\n");
   run("reads, then MFMAs; no barrier", feed_kernel<0, 0>, 8, 32, 2000, out, clk);
   run("reads, then MFMAs; barrier per slice", feed_kernel<0, 1>, 8, 32, 2000, out, clk);
   run("reads one slice ahead; no barrier", feed_kernel<1, 0>, 8, 32, 2000, out, clk);
   run("reads one slice ahead; barrier per slice", feed_kernel<1, 1>, 8, 32, 2000, out, clk);
+  printf("-- the same wave tile on v_mfma_i32_32x32x32_i8: 12 ds_read_b128 + 32 xor + 16 MFMA per wave and K slice --\n");
+  run("32x32x32: reads, then MFMAs; no barrier", feed32_kernel<0, 0>, 8, 16, 2000, out, clk, 65536);
+  run("32x32x32: reads, then MFMAs; barrier per slice", feed32_kernel<0, 1>, 8, 16, 2000, out, clk, 65536);
+  run("32x32x32: reads one slice ahead; no barrier", feed32_kernel<1, 0>, 8, 16, 2000, out, clk, 65536);
+  run("32x32x32: reads one slice ahead; barrier per slice", feed32_kernel<1, 1>, 8, 16, 2000, out, clk, 65536);
+  printf("-- LDS read rate: conflict-free ds_read_b128 back to back, one workgroup per compute unit --\n");
+  for (int w = 4; w <= 16; w *= 2) {
+    const int iters = 4000;
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    CK(hipFuncSetAttribute((const void *)ldsbw_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024));
+    hipLaunchKernelGGL(ldsbw_kernel, dim3(g_cus), dim3(64 * w), 100 * 1024, 0, out, clk, iters);
+    CK(hipEventRecord(e0, 0));
+    hipLaunchKernelGGL(ldsbw_kernel, dim3(g_cus), dim3(64 * w), 100 * 1024, 0, out, clk, iters);
+    CK(hipEventRecord(e1, 0));
+    CK(hipDeviceSynchronize());
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    long long h[2];
+    CK(hipMemcpy(h, clk, 16, hipMemcpyDeviceToHost));
+    const double mhz = (double)h[0] / (h[1] / 100.0);
+    printf("ds_read_b128, %d waves/SIMD: %.1f bytes per cycle per compute unit (%4.0f MHz)\n", w / 4,
+           (double)w * iters * 8 * 1024 / (ms * 1e-3 * mhz * 1e6), mhz);
+  }
   printf("-- vector ALU: cycles per wave64 instruction per SIMD (one workgroup per compute unit, independent chains) --\n");
   run_valu<0>("v_dot4c_i32_i8", out, clk);
   run_valu<1>("v_dot4_i32_i8", out, clk);

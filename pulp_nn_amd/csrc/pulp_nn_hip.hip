@@ -16,6 +16,7 @@
 #include "../../include/32bit/pulp_nn_kernels.h"
 #endif
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 
@@ -23,7 +24,7 @@
 #include "depthwise.h"
 #include "dwpw_fused.h"
 #include "igemm.h"
-#include "igemm_dma.h"
+#include "igemm_ring.h"
 #include "linear_skinny.h"
 #include "pool.h"
 #include "pw_stream.h"
@@ -146,28 +147,41 @@ bool raise_lds_limit(size_t lds)
   return true;
 }
 
-// 256 x 256 tiles fed by LDS-direct loads (igemm_dma.h).  Returns false if the kernel cannot be launched.
-bool launch_igemm_dma(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+// 256 x 256 tiles of persistent workgroups fed by LDS-direct loads (igemm_ring.h).  Returns false if the shape
+// does not qualify or the kernel cannot be launched (the caller then uses the tiled kernel).
+bool launch_igemm_ring(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
 {
-  g.tiles_n = (g.N + 255) / 256;
-  g.tiles_total = ((g.M + 255) / 256) * g.tiles_n;
+  typedef IgrShape<4> S;
+  // K: at least as many sub-slices as ring stages; below 2^16, so that accumulator and correction term each
+  // fit 32 bits (the epilogue adds them in 64-bit arithmetic in the 64-bit build)
+  if (g.Ci % 64 || g.K < 64 * S::NS || g.K >= 65536 || g.N % 16 || !aligned(g.out, 16) || mode == EPI_OUT32) return false;
+  g.tiles_n = (g.N + S::BN - 1) / S::BN;
+  g.tiles_total = ((g.M + IGR_BM - 1) / IGR_BM) * g.tiles_n;
+  // the grid: a multiple of 8 * tiles_n workgroups (a workgroup keeps its channel range, an XCD gets whole
+  // pixel tiles), at most one per compute unit and no more than there are tiles
+  const int unit = 8 * g.tiles_n;
+  const int grid_n = (int)(std::min<long long>(num_cus(), g.tiles_total) / unit) * unit;
+  if (grid_n <= 0) return false;
   conv_geom_divs(g);
-  g.vec_store = (g.N % 16 == 0) && aligned(g.out, 16);
-  g.nt = 0;
-  const size_t lds = (size_t)igd_lds_bytes();
-  const dim3 grid(g.tiles_total), block(IGD_THREADS);
+  g.cpt = g.Ci / 64;
+  g.d_cpt = fastdiv_make((unsigned)g.cpt);
+  g.d_kx = fastdiv_make((unsigned)g.kx);
+  g.vec_store = 1;
+  g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
+  const size_t lds = (size_t)S::lds_bytes();
+  const dim3 grid(grid_n), block(S::THREADS);
   switch (mode) {
     case EPI_BN:
-      if (!raise_lds_limit<igemm_dma_kernel<EPI_BN>>(lds)) return false;
-      hipLaunchKernelGGL(igemm_dma_kernel<EPI_BN>, grid, block, lds, s, g, e);
+      if (!raise_lds_limit<igemm_ring_kernel<EPI_BN, 4>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_ring_kernel<EPI_BN, 4>), grid, block, lds, s, g, e);
       break;
     case EPI_MULT:
-      if (!raise_lds_limit<igemm_dma_kernel<EPI_MULT>>(lds)) return false;
-      hipLaunchKernelGGL(igemm_dma_kernel<EPI_MULT>, grid, block, lds, s, g, e);
+      if (!raise_lds_limit<igemm_ring_kernel<EPI_MULT, 4>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_ring_kernel<EPI_MULT, 4>), grid, block, lds, s, g, e);
       break;
     default:
-      if (!raise_lds_limit<igemm_dma_kernel<EPI_RAW>>(lds)) return false;
-      hipLaunchKernelGGL(igemm_dma_kernel<EPI_RAW>, grid, block, lds, s, g, e);
+      if (!raise_lds_limit<igemm_ring_kernel<EPI_RAW, 4>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_ring_kernel<EPI_RAW, 4>), grid, block, lds, s, g, e);
       break;
   }
   return true;
@@ -189,8 +203,8 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   // L2 -> LDS bytes per multiply of the 128 x 128 tile
   const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
   if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) {
-    // whole 128-byte lines per pixel and K slice: operands go HBM/L2 -> LDS without passing through registers
-    if (g.Ci % 128 == 0 && mode != EPI_OUT32 && launch_igemm_dma(mode, g, e, s)) return;
+    // operands go HBM/L2 -> LDS without passing through registers, persistent workgroups
+    if (launch_igemm_ring(mode, g, e, s)) return;
     launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
   } else
   // 128 px x 64 ch while 128 x 128 tiles would give a CU at most one workgroup: twice the workgroups to

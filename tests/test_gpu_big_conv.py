@@ -1,8 +1,10 @@
-"""GPU parity of the large-tile convolution path (256 x 256 tiles fed by LDS-direct loads).
+"""GPU parity of the large-tile convolution path (persistent workgroups on 256 x 256 tiles fed by LDS-direct loads).
 
-That path is taken by convolutions with input channels a multiple of 128, more than 128 output channels and
-at least two 256 x 256 tiles per compute unit; these geometries are sized to reach it and to exercise its
-edges (channel tail, pixel tail, padding on every side, stride 2, every epilogue branch, both widths)."""
+That path is taken by convolutions with input channels a multiple of 64, more than 128 output channels (a multiple
+of 16), K of at least 256 bytes and at least two 256 x 256 tiles per compute unit; these geometries are sized to reach
+it and to exercise its edges (channel tail, pixel tail, padding on every side, stride 2, several channel tiles, an
+odd number of K sub-slices, the shortest K, every epilogue branch, both widths).  One geometry (136 channels) stays
+on the tiled kernel of the same tile size."""
 import numpy as np
 import pytest
 
@@ -17,6 +19,9 @@ GEOMS = [
     (140, 31, 33, 128, 192, 3, 3, (1, 0, 1, 0), (1, 1)),    # channel tail (192 of a 256 tile), odd sizes, asymmetric pads
     (150, 60, 62, 128, 136, 3, 3, (0, 1, 0, 1), (2, 2)),    # stride 2, pads bottom / right only
     (140, 32, 32, 256, 256, 1, 3, (0, 0, 1, 1), (1, 1)),    # 1 x 3 filter, K = 768
+    (84, 40, 40, 64, 256, 3, 3, (1, 1, 1, 1), (1, 1)),      # 64 input channels: one K sub-slice per tap, nine in all (odd)
+    (70, 48, 48, 192, 512, 3, 3, (1, 1, 1, 1), (1, 1)),     # two channel tiles per pixel tile, three sub-slices per tap
+    (262, 23, 23, 320, 256, 1, 1, (0, 0, 0, 0), (1, 1)),    # K = 320: five sub-slices, one more than the ring has stages
 ]
 FLAGS = [(1, 1), (1, 0), (0, 0), (0, 1)]
 
