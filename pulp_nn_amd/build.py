@@ -38,21 +38,25 @@ def build(bn_bits, verbose=False):
     return out
 
 
-def tool_path():
-    return os.path.join(LIBDIR, "mfma_ceiling")
+TOOLS = ("mfma_ceiling", "conv_phases")
 
 
-def build_tool(verbose=False):
-    """The matrix-core yardstick (csrc/mfma_ceiling.hip): a stand-alone executable, no part of the libraries."""
+def tool_path(name="mfma_ceiling"):
+    return os.path.join(LIBDIR, name)
+
+
+def build_tool(name="mfma_ceiling", verbose=False):
+    """The measurement tools: the matrix-core yardstick (csrc/mfma_ceiling.hip) and the phase / ablation trace of
+    the large convolution (csrc/conv_phases.hip).  Stand-alone executables, no part of the libraries."""
     os.makedirs(LIBDIR, exist_ok=True)
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", os.path.join(CSRC, "mfma_ceiling.hip"), "-o", tool_path()]
+           "-packed-fp32-ops", os.path.join(CSRC, name + ".hip"), "-o", tool_path(name)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + res.stdout)
-    return tool_path()
+    return tool_path(name)
 
 
 def demo_path():
@@ -77,10 +81,10 @@ def build_demo(verbose=False):
 
 def build_all(verbose=False):
     from concurrent.futures import ThreadPoolExecutor
-    with ThreadPoolExecutor(3) as ex:
+    with ThreadPoolExecutor(4) as ex:
         libs = [ex.submit(build, b, verbose) for b in (32, 64)]
-        tool = ex.submit(build_tool, verbose)
-        out = [f.result() for f in libs] + [tool.result()]
+        tools = [ex.submit(build_tool, t, verbose) for t in TOOLS]
+        out = [f.result() for f in libs] + [f.result() for f in tools]
     return out + [build_demo(verbose)]
 
 
