@@ -82,7 +82,9 @@ void pulp_nn_hip_depthwise_hwc(const unsigned char *Im_in, const signed char *bi
  * parameters (dw_*: the depthwise layer's; pw_*: the pointwise layer's, pw_weight[ch_out][ch]);
  * the intermediate tensor is never written.  k / lambda arrays are int32_t or int64_t as the
  * build expects.  Supported: dim_im_in_x in {64, 32, 16, 8} (and 4 with stride 1), ch in
- * {16, 32} or a multiple of 64 up to 1024, ch_out a multiple of 16, output rows a multiple of
+ * {16, 32} or a multiple of 64 up to 1024, ch_out a multiple of 16 and at most 1024 per
+ * workgroup (small layers are split over several workgroups by output channels, so more can
+ * pass; a large batch with ch_out > 1024 cannot), output rows a multiple of
  * the rows a wave takes at once (2 to 8, times 64 / ch for ch < 64), 16-byte aligned pointwise
  * weights and output.  Anything else sets PULP_NN_HIP_ERR_UNSUPPORTED and queues nothing:
  * make the two calls instead. */
@@ -133,6 +135,10 @@ void pulp_nn_hip_dw_pw_chain_hwc(const unsigned char *Im_in, unsigned char *Im_o
  * result points to two 64-bit words in DEVICE memory, written on the stream:
  * result[0] = max |acc * k[c]| (64-bit wrapping product, as the 64-bit tree forms it),
  * result[1] = max(floor(log2(result[0])) - 7, 0), and 0 for a layer whose maximum is 0.
+ * The 32-bit build reports the same unwrapped 64-bit magnitude, although its layers form
+ * acc * k in int32 (32bit/src/pulp_nn_utils.c:35-45): result[0] >= 2^31 means that the
+ * layer's product wraps on this batch and result[1] does not describe it; callers check
+ * result[0] < 2^31 there.
  * k is an int32_t or int64_t array as the build expects.  The geometry arguments have the
  * meaning they have in pulp_nn_conv_Ho_parallel (a pointwise layer is a 1x1 kernel with
  * stride 1 and no padding; a linear layer is a pointwise layer on a 1x1 image) and in

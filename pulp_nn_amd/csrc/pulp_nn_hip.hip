@@ -265,7 +265,7 @@ void launch_smallk(int mode, bool rows, ConvGeom &g, const EpiArgs &e, hipStream
 
 // Launches one instantiation; raises its dynamic-LDS limit above the default 64 KB as needed.
 template <auto KERN>
-void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t lds, hipStream_t s)
+bool launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t lds, hipStream_t s)
 {
   // (raising the limit twice from two host threads is harmless; the mutex keeps the cached value
   // from running ahead of the attribute)
@@ -274,11 +274,15 @@ void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t 
   if (lds > limit.load(std::memory_order_acquire)) {
     std::lock_guard<std::mutex> lock(mu);
     if (lds > limit.load(std::memory_order_relaxed)) {
-      (void)hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (hipFuncSetAttribute((const void *)KERN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
       limit.store(lds, std::memory_order_release);
     }
   }
   hipLaunchKernelGGL(KERN, grid, block, lds, s, g, e);
+  return true;
 }
 
 // Two shapes of the streaming kernel: 16 waves taking 16 pixels per step for launches
@@ -287,31 +291,30 @@ void launch_pw(const PwGeom &g, const EpiArgs &e, dim3 grid, dim3 block, size_t 
 // per step otherwise (half the LDS reads per pixel, and the 128-register budget of the
 // 16-wave shape is too small for K = 256).
 template <int TN, int NP, int KS, int TM, int NW>
-void launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
+bool launch_pw_stream_mode(int mode, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds, hipStream_t s)
 {
   dim3 block(64 * NW);
   switch (mode) {
-    case EPI_BN: launch_pw<pw_stream_kernel<TN, KS, NP, EPI_BN, false, TM, NW>>(g, e, grid, block, lds, s); break;
+    case EPI_BN: return launch_pw<pw_stream_kernel<TN, KS, NP, EPI_BN, false, TM, NW>>(g, e, grid, block, lds, s);
     case EPI_MULT:
-      if (e.shift >= 16) launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, true, TM, NW>>(g, e, grid, block, lds, s);
-      else launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, false, TM, NW>>(g, e, grid, block, lds, s);
-      break;
-    default: launch_pw<pw_stream_kernel<TN, KS, NP, EPI_RAW, false, TM, NW>>(g, e, grid, block, lds, s); break;
+      if (e.shift >= 16) return launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, true, TM, NW>>(g, e, grid, block, lds, s);
+      return launch_pw<pw_stream_kernel<TN, KS, NP, EPI_MULT, false, TM, NW>>(g, e, grid, block, lds, s);
+    default: return launch_pw<pw_stream_kernel<TN, KS, NP, EPI_RAW, false, TM, NW>>(g, e, grid, block, lds, s);
   }
 }
 
 template <int TN, int NP>
-void launch_pw_stream_ks(int mode, int ks, bool wide, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds,
+bool launch_pw_stream_ks(int mode, int ks, bool wide, const PwGeom &g, const EpiArgs &e, dim3 grid, size_t lds,
                          hipStream_t s)
 {
   if (ks == 1) {
-    if (wide) launch_pw_stream_mode<TN, NP, 1, 1, 16>(mode, g, e, grid, lds, s);
-    else launch_pw_stream_mode<TN, NP, 1, 2, 8>(mode, g, e, grid, lds, s);
+    if (wide) return launch_pw_stream_mode<TN, NP, 1, 1, 16>(mode, g, e, grid, lds, s);
+    return launch_pw_stream_mode<TN, NP, 1, 2, 8>(mode, g, e, grid, lds, s);
   } else if (ks == 2) {
-    if (wide) launch_pw_stream_mode<TN, NP, 2, 1, 16>(mode, g, e, grid, lds, s);
-    else launch_pw_stream_mode<TN, NP, 2, 2, 8>(mode, g, e, grid, lds, s);
+    if (wide) return launch_pw_stream_mode<TN, NP, 2, 1, 16>(mode, g, e, grid, lds, s);
+    return launch_pw_stream_mode<TN, NP, 2, 2, 8>(mode, g, e, grid, lds, s);
   } else {
-    launch_pw_stream_mode<TN, NP, 4, 2, 8>(mode, g, e, grid, lds, s);
+    return launch_pw_stream_mode<TN, NP, 4, 2, 8>(mode, g, e, grid, lds, s);
   }
 }
 
@@ -352,13 +355,13 @@ bool try_pw_stream(int mode, const uint8_t *in, const int8_t *w, const int8_t *b
   // every CU takes part there, and staging the weights per workgroup no longer pays
   if (2 * need < num_cus()) return false;
   dim3 grid(blocks);
-  if (tn == 1) launch_pw_stream_ks<1, 1>(mode, ks, wide, g, e, grid, lds, s);
-  else if (tn == 2) launch_pw_stream_ks<2, 1>(mode, ks, wide, g, e, grid, lds, s);
-  else if (np == 1) launch_pw_stream_ks<4, 1>(mode, ks, wide, g, e, grid, lds, s);
-  else if (np == 2) launch_pw_stream_ks<4, 2>(mode, ks, wide, g, e, grid, lds, s);
-  else if (np == 3) launch_pw_stream_ks<4, 3>(mode, ks, wide, g, e, grid, lds, s);
-  else launch_pw_stream_ks<4, 4>(mode, ks, wide, g, e, grid, lds, s);
-  return true;
+  // (false also if the kernel's LDS limit cannot be raised: the caller then uses the tiled kernel)
+  if (tn == 1) return launch_pw_stream_ks<1, 1>(mode, ks, wide, g, e, grid, lds, s);
+  if (tn == 2) return launch_pw_stream_ks<2, 1>(mode, ks, wide, g, e, grid, lds, s);
+  if (np == 1) return launch_pw_stream_ks<4, 1>(mode, ks, wide, g, e, grid, lds, s);
+  if (np == 2) return launch_pw_stream_ks<4, 2>(mode, ks, wide, g, e, grid, lds, s);
+  if (np == 3) return launch_pw_stream_ks<4, 3>(mode, ks, wide, g, e, grid, lds, s);
+  return launch_pw_stream_ks<4, 4>(mode, ks, wide, g, e, grid, lds, s);
 }
 
 // Shared body of the six convolution entry points.
@@ -751,7 +754,10 @@ void calib_common(const char *fn, CalibGeom &g, unsigned long long *partial, uns
   if (g.W <= 0 || g.H <= 0 || g.Ci <= 0 || g.Wo <= 0 || g.Ho <= 0 || g.Co <= 0 || g.kx <= 0 || g.ky <= 0 || g.sx <= 0 ||
       g.sy <= 0)
     return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "zero dimension");
-  g.total = (long long)g_batch * g.Ho * g.Wo * g.Co;
+  // batch * Ho * Wo * Co can pass 2^63 (batch up to 2^31, the dimensions up to 2^16 each): bound it before it is formed
+  const unsigned long long per_image = (unsigned long long)g.Ho * g.Wo * g.Co;  // < 2^48
+  if ((unsigned long long)g_batch > (1ull << 47) / per_image) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
+  g.total = (long long)((unsigned long long)g_batch * per_image);
   g.in_img = (long long)g.H * g.W * g.Ci;
   const unsigned long long slots = ((unsigned long long)g.total + CALIB_CHUNK - 1) / CALIB_CHUNK;
   if (slots > 0x7fffffffull) return set_error(PULP_NN_HIP_ERR_ARGUMENT, fn, "batch too large");
@@ -1113,6 +1119,9 @@ static void dwpw_common(const char *fn, const unsigned char *Im_in, unsigned cha
   // few pixel tiles: several workgroups share one, each with a part of the output channels (and its own copy of stage 1)
   g.nsplit = 1;
   while (tiles * g.nsplit < num_cus() && g.nsplit * 2 <= nbt) g.nsplit *= 2;
+  // (the kernel stages the pointwise constants of at most 1024 channels per workgroup)
+  if (((nbt + g.nsplit - 1) / g.nsplit) * 64 > 1024)
+    return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "more than 1024 output channels per workgroup: call the depthwise and the pointwise layer separately");
   size_t lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(((nbt + g.nsplit - 1) / g.nsplit) * 64);
   if (n_blocks > 1) {
     // Several blocks: the output of one is the next one's input and stays in LDS, so a tile has to be whole images

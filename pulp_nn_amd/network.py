@@ -17,7 +17,8 @@ produces the tensor called like the layer.  Activations are HWC uint8, batch out
                 pointwise layer that is the only reader of the depthwise result, the two run
                 as one launch (pulp_nn_hip_dw_pw_hwc) and the depthwise result is not
                 materialised: Runner(..., fuse_blocks=True) for every such pair, False for none,
-                "auto" (the default) for planes up to 16 pixels wide, where it is not slower
+                "auto" (the default) where it is not slower: as Runner.tune() measured it on the
+                batch at hand, else for blocks whose output plane is 8 x 8 pixels
   maxpool       kernel (kx,ky), strides, pads, out_hw      -> pulp_nn_maxpool
   avgpool       kernel, strides, pads, out_hw, lam, shift, add, requant -> pulp_nn_avgpool
   add           in = (a, b), m1, m2, shift                 -> pulp_nn_add
@@ -85,6 +86,7 @@ class Runner:
         self.nn, self.layers, self.batch, self.torch = nn, layers, batch, torch
         self.fused, self.unfused = fused, set()
         self.fuse_blocks, self.unfused_blocks, self.launches = fuse_blocks, set(), 0
+        self.block_choice = {}   # layer index of a depthwise layer -> run it and its pointwise layer as one launch (tune())
         # runs of depthwise + pointwise blocks of one shape as one launch each (pulp_nn_hip_dw_pw_chain_hwc)
         self.chain_blocks, self.unchained = bool(chain_blocks and fused and fuse_blocks), set()
         self.shapes = infer_shapes(layers, input_shape)
@@ -217,12 +219,19 @@ class Runner:
         L, N = self.layers[i], self.layers[i + 1]
         if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
             return False
-        # "auto": only where the single launch is not slower than the two.  Measured on MI355X at batch 256
-        # (kernel times of the MobileNet chain's blocks): 16-pixel planes at stride 2 (11.2 us against 5.9 + 6.4) and
-        # 8-pixel planes at stride 1 (11.8 against 5.4 + 7.1) gain; 16-pixel planes at stride 1 (17.8 against
-        # 7.9 + 8.2), 8-pixel planes at stride 2, 4-pixel planes and everything wider lose.
-        if policy and self.fuse_blocks == "auto" and (self.shapes[L["in"]][1], L["strides"][0]) not in ((16, 2), (8, 1)):
-            return False
+        # "auto": only where the single launch is not slower than the two.  Runner.tune() times both forms of every
+        # such block on the batch at hand and records the faster one in block_choice.  Without that measurement the
+        # rule is the shape of the fused kernel's work: it pays where an image's output plane is 8 x 8 pixels, so
+        # that one workgroup takes whole images and each of its eight waves one item of the depthwise stage (on
+        # MI355X at batch 256: 11.2 us against 5.9 + 6.4 for 16-pixel planes at stride 2, 11.8 against 5.4 + 7.1
+        # for 8-pixel planes at stride 1); larger output planes split an image over workgroups that each run the
+        # whole load -> depthwise -> MFMA -> store chain, smaller ones leave waves without an item.
+        if policy and self.fuse_blocks == "auto":
+            if i in self.block_choice:
+                if not self.block_choice[i]:
+                    return False
+            elif tuple(self.shapes[L["name"]][:2]) != (8, 8):
+                return False
         if L["op"] != "depthwise" or N["op"] != "pointwise" or N["in"] != L["name"]:
             return False
         sx, sy = L["strides"]
@@ -321,7 +330,57 @@ class Runner:
             nn.calib_conv(cur, P.get("bias"), P["w"], P["k"], W, H, Cc, Wo, Ho, Co, kx, ky, pt, pl, sx, sy, ws, nbytes, res)
         nn.sync()
         m, shift = (int(v) for v in res.cpu().numpy().view(np.uint64))
+        if nn.bn_bits == 32 and m >= 2 ** 31:
+            # the 32-bit tree forms acc * k in int32 (pulp_nn_utils.c:35-45): the layer's product wraps on this batch,
+            # and no out_shift derived from the unwrapped maximum describes what the layer computes
+            raise ValueError("layer %s: max |acc * k| = %d does not fit int32; the 32-bit batch-norm product wraps "
+                             "(use smaller k or the 64-bit library)" % (L["name"], m))
         return m, shift
+
+    def tune(self, x, reps=20):
+        """Times every depthwise + pointwise block that can be one launch (and is not part of a chained run) both
+        ways on this batch and keeps the faster form (fuse_blocks="auto" then follows these choices instead of the
+        shape rule).  Needs every out_shift (run calibrate() first).  Returns {depthwise layer name: fused?}."""
+        torch = self.torch
+        self.nn.set_batch(self.batch)
+        tensors = {"input": x}
+        self.run(x)
+        for L in self.layers:
+            tensors[L["name"]] = self.act[L["name"]]
+        self.nn.sync()
+
+        def timed(fn):
+            fn()
+            self.nn.sync()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            self.nn.sync()
+            return e0.elapsed_time(e1) / reps
+
+        chosen = {}
+        i = 0
+        while i < len(self.layers):
+            n = self._chain_length(i) if self.chain_blocks else 0
+            if n >= 2:
+                i += 2 * n
+                continue
+            if self._block_fusable(i, policy=False):
+                ok = self._queue_block(i, tensors)   # False: the library has no fused kernel for this geometry
+                if ok:
+                    t_fused = timed(lambda: self._queue_block(i, tensors))
+                    t_split = timed(lambda: (self._queue(i, tensors), self._queue(i + 1, tensors)))
+                    self.block_choice[i] = t_fused <= t_split
+                else:
+                    self.block_choice[i] = False
+                chosen[self.layers[i]["name"]] = self.block_choice[i]
+                i += 2
+                continue
+            i += 1
+        self.nn.sync()
+        return chosen
 
     def calibrate(self, x, force=False):
         """Runs the chain on x and gives every batch-norm layer without an out_shift (all of them with

@@ -26,6 +26,7 @@ GEOMS = [
     (4, 16, 16, 192, 80, 1),     # three channel groups, output channels not a multiple of 64
     (300, 8, 8, 64, 16, 1),      # many small images, a single 16-channel output group
     (9, 8, 16, 320, 96, 2),      # H = 8, W = 16, five K slices (two passes over the weights)
+    (4, 8, 8, 64, 2048, 1),      # 2048 output channels: legal because so few images are split over workgroups by channels
 ]
 FLAGS = [((1, 1), (1, 1)), ((1, 0), (1, 1)), ((1, 1), (1, 0)), ((0, 0), (0, 0)), ((2, 0), (0, 1))]
 
@@ -104,6 +105,18 @@ def test_fused_block_rejects_what_it_cannot_do():
     assert err.value.code == 2
     with pytest.raises(PulpNNError):                                           # wrong output size
         L.dw_pw_hwc(x, out, 16, 16, 64, 15, 16, 64, 1, w9, None, None, None, 300, 15, 1, 0, pw, None, None, None, 300, 15, 1, 0)
+    # more than 1024 output channels in one workgroup: a batch large enough that the tiles are not split by channels
+    B = 1024
+    xb = torch.zeros((B, 8, 8, 64), dtype=torch.uint8, device="cuda")
+    ob = torch.zeros((B, 8, 8, 2048), dtype=torch.uint8, device="cuda")
+    pwb = torch.zeros((2048, 64), dtype=torch.int8, device="cuda")
+    L.set_batch(B)
+    try:
+        with pytest.raises(PulpNNError) as err:
+            L.dw_pw_hwc(xb, ob, 8, 8, 64, 8, 8, 2048, 1, w9, None, None, None, 300, 15, 1, 0, pwb, None, None, None, 300, 15, 1, 0)
+        assert err.value.code == 2
+    finally:
+        L.set_batch(1)
 
 
 # ---- several blocks of one shape in one launch (pulp_nn_hip_dw_pw_chain_hwc) --------------------------------------

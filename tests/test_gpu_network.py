@@ -158,6 +158,57 @@ def test_resnet_style_block_batch256(bn_bits):
     assert out.data_ptr() == runner.act["fc"].data_ptr()
 
 
+def test_fusion_choice_on_a_table_that_is_not_a_mobilenet():
+    """The ResNet-style block with two depthwise + pointwise pairs put in front of its tail: the runner's default
+    rule and the timed choice of tune() each pick one form per pair, and either way every layer equals the oracle."""
+    r = rng_for(22500)
+    B, C = 64, 64
+    layers = resnet_block(r, C, 32)[:5]
+
+    def bnp(n):
+        return dict(k=r.integers(256, 1025, n), lam=r.integers(-2 ** 16, 2 ** 16 + 1, n), relu=1, bn=1, shift=None)
+
+    layers += [
+        dict(op="depthwise", name="dw1", **{"in": "sum"}, w=rand_s8(r, (C, 3, 3)), bias=rand_s8(r, (C,)), pads=(1, 1, 1, 1),
+             strides=(1, 1), **bnp(C)),                                   # 16 x 16 planes at stride 1: 16 x 16 out
+        dict(op="pointwise", name="pw1", **{"in": "dw1"}, w=rand_s8(r, (2 * C, 1, 1, C)), bias=rand_s8(r, (2 * C,)), **bnp(2 * C)),
+        dict(op="depthwise", name="dw2", **{"in": "pw1"}, w=rand_s8(r, (2 * C, 3, 3)), bias=rand_s8(r, (2 * C,)),
+             pads=(1, 1, 1, 1), strides=(2, 2), **bnp(2 * C)),            # 16 x 16 planes at stride 2: 8 x 8 out
+        dict(op="pointwise", name="pw2", **{"in": "dw2"}, w=rand_s8(r, (2 * C, 1, 1, 2 * C)), bias=None, **bnp(2 * C)),
+        dict(op="avgpool", name="gap", **{"in": "pw2"}, kernel=(4, 4), strides=(4, 4), out_hw=(2, 2), lam=3, shift=1, add=5,
+             requant=1),
+        dict(op="linear", name="fc", **{"in": "gap"}, w=rand_s8(r, (50, 2 * 2 * 2 * C)), bias=rand_s8(r, (50,)), **bnp(50)),
+    ]
+    x = rand_u8(r, (B, 32, 32, 3))
+    L = nn(32)
+    runner = network.Runner(L, layers, (32, 32, 3), B)
+    xd = torch.from_numpy(x).cuda()
+    runner.calibrate(xd)
+    i1, i2 = [i for i, Ld in enumerate(layers) if Ld["op"] == "depthwise"]
+    # the rule: one launch for the pair with an 8 x 8 output plane only
+    assert not runner._block_fusable(i1) and runner._block_fusable(i2)
+    runner.run(xd)
+    L.sync()
+    assert runner.launches == len(layers) - 1
+    want = net_oracle.forward(layers, runner.shapes, x, 32, keep=True)
+    check = [Ld["name"] for Ld in layers if Ld["name"] != "dw2"]          # dw2 is not materialised when its pair is fused
+    for name in check:
+        assert_same(runner.act[name].cpu().numpy(), want[name], "rule-based path, layer %s" % name)
+    # the timed choice: whatever it picks, the results stay those of the oracle
+    chosen = runner.tune(xd)
+    assert set(chosen) == {"dw1", "dw2"} and all(isinstance(v, bool) for v in chosen.values())
+    for Ld in layers:
+        runner.act[Ld["name"]].zero_()
+    runner.run(xd)
+    L.sync()
+    L.set_batch(1)
+    assert runner.launches == len(layers) - sum(chosen.values())
+    for Ld in layers:
+        fused_away = Ld["op"] == "depthwise" and chosen[Ld["name"]]
+        if not fused_away:
+            assert_same(runner.act[Ld["name"]].cpu().numpy(), want[Ld["name"]], "timed path, layer %s" % Ld["name"])
+
+
 @pytest.mark.parametrize("case", [
     # B, H, W, C, kernel(kx,ky), strides(sx,sy), pads(t,b,l,r), out_hw
     (2, 32, 32, 64, (3, 3), (2, 2), (1, 1, 1, 1), (16, 16)),     # ResNet stem pooling

@@ -1,9 +1,12 @@
 """The allocation-free calibration entry point (pulp_nn_hip_calib_conv_static) against the
-workspace one, through the C ABI: two calls in a row, the second on a smaller input."""
+workspace one and against the exact integers of the layer's accumulators, through the C ABI:
+two calls in a row, the second on a smaller input; and the device's free memory does not move
+across such a call."""
 import numpy as np
 import pytest
 import torch
 
+import net_oracle
 from gpu_helpers import bn_dev, dev, nn, rand_s8, rand_u8, rng_for
 
 pytestmark = pytest.mark.gpu
@@ -43,8 +46,34 @@ def test_static_scratch_calibration_matches_workspace_calibration(bn_bits):
         a, s = both(L, bn_bits, x, w, b, k, (H, W, Ci, H, W, Co, kx, ky, pt, pl, sx, sy))
         np.testing.assert_array_equal(s, a)
         assert a[0] > 0
+        # the static path against the layer's accumulators in exact integers (numpy)
+        layer = dict(op="conv", w=w, bias=b, k=k, pads=(pt, pt, pl, pl), strides=(sx, sy))
+        want = net_oracle.absmax(layer, x, (H, W))
+        assert int(s[0]) == want and int(s[1]) == net_oracle.shift_from(want)
         results.append(int(a[0]))
     assert results[1] < results[0]
+
+
+def test_static_scratch_calibration_allocates_nothing():
+    r = rng_for(24100)
+    L = nn(32)
+    B, H, W, Ci, Co = 6, 20, 20, 8, 16
+    x, w, b = rand_u8(r, (B, H, W, Ci)), rand_s8(r, (Co, 3, 3, Ci)), rand_s8(r, (Co,))
+    xd, wd, bd, kd = dev(x), dev(w), dev(b), bn_dev(r.integers(256, 1025, Co), 32)
+    res = torch.zeros(2, dtype=torch.int64, device="cuda")
+    L.set_batch(B)
+    try:
+        L.calib_conv_static(xd, bd, wd, kd, W, H, Ci, W, H, Co, 3, 3, 1, 1, 1, 1, res)   # first call on this device: looks the array up
+        L.sync()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for _ in range(3):
+            L.calib_conv_static(xd, bd, wd, kd, W, H, Ci, W, H, Co, 3, 3, 1, 1, 1, 1, res)
+        L.sync()
+        assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
+    finally:
+        L.set_batch(1)
+    assert int(res[0]) > 0
 
 
 def test_static_scratch_calibration_rejects_a_layer_beyond_its_slots():
