@@ -9,9 +9,13 @@ multiplier requantisation + ReLU), the configuration the headline metric is
 quoted on.  Inputs are resident in HBM before the timed region; successive steps
 rotate through enough buffer sets (> 256 MB in total) that the Infinity Cache
 cannot hold them.  A timed region is exactly K steps between two device
-synchronisations; because K steps of a 17 us kernel are far too short to time
-once, the region is repeated (at least 5 times and until 5 ms have been timed)
-and the median is reported.  The last line printed is the JSON record.
+synchronisations.  K steps of a 17 us kernel are far too short to time once, and
+the shader clock of this GPU settles only after some 10 ms of continuous work (a
+burst of a few launches of the MFMA-bound convolution runs up to a third slower
+than the same launches in a long run), so regions are repeated back to back, at
+least 10 times and until 60 ms have been timed.  The median over the regions is
+the reported value; the first region, minimum, 10th and 90th percentile go into
+the record next to it ("timing").  The last line printed is the JSON record.
 
 Besides the headline workload the record carries, under "layers", the other
 single-layer configurations (3x3 conv at batch 256, depthwise 3x3 stride 1 and 2
@@ -64,6 +68,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--quick", action="store_true", help="time 6 ms per workload instead of 60 (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus 1): every layer is independent per image, so "
@@ -85,10 +90,11 @@ def main():
     def t(a):
         return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
-    def time_launches(fn, steps, warmup, min_ms=5.0, min_repeats=5, max_repeats=400):
+    def time_launches(fn, steps, warmup, min_ms=None, min_repeats=10, max_repeats=4000):
         """fn(i) queues one step on torch's current stream (the library's stream).  Times regions of exactly
-        `steps` steps, each between two synchronisations; returns the medians of (wall ms per step, device ms
-        per step from HIP events) and the number of regions."""
+        `steps` steps, each between two synchronisations, one after the other; returns (median wall ms per step,
+        median device ms per step from HIP events, timing summary)."""
+        min_ms = (6.0 if args.quick else 60.0) if min_ms is None else min_ms
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
@@ -107,7 +113,19 @@ def main():
             walls.append((t1 - t0) * 1e3 / steps)
             devs.append(e0.elapsed_time(e1) / steps)
             timed += e0.elapsed_time(e1)
-        return statistics.median(walls), statistics.median(devs), len(walls)
+        srt = sorted(devs)
+
+        def pct(q):
+            return srt[min(len(srt) - 1, int(q * len(srt)))]
+
+        summary = {"regions": len(devs), "steps_per_region": steps, "timed_ms": round(timed, 1),
+                   "device_us_per_step": {"first_region": round(devs[0] * 1e3, 2), "min": round(srt[0] * 1e3, 2),
+                                          "p10": round(pct(0.10) * 1e3, 2), "median": round(statistics.median(devs) * 1e3, 2),
+                                          "p90": round(pct(0.90) * 1e3, 2),
+                                          "median_after_first_10ms": round(statistics.median(
+                                              devs[min(len(devs) - 1, next((n for n in range(len(devs)) if sum(devs[:n + 1]) * steps >= 10.0),
+                                                                            len(devs) - 1)):]) * 1e3, 2)}}
+        return statistics.median(walls), statistics.median(devs), summary
 
     def rotating(nbytes):
         """How many buffer sets make the rotation exceed the 256 MB Infinity Cache twice over."""
@@ -123,7 +141,10 @@ def main():
             r.update(achieved=round(nbytes / sec / 1e9, 1), peak=PEAK_HBM / 1e9, unit="GB/s",
                      frac=round(nbytes / sec / PEAK_HBM, 4))
         r["algorithmic_bytes_per_launch"] = nbytes
+        # (from the committed counter summary, looked up by the kernel this layer is expected to dispatch to; null if
+        # that kernel has no line there)
         r["traffic"] = traffic_for(traffic, kernel.split("(")[0].strip())
+        r["traffic_measured_in_this_run"] = False
         return r
 
     # ---- headline: config 1 -------------------------------------------------
@@ -143,7 +164,7 @@ def main():
         L.pulp_nn_pointwise_HoWo_parallel(xs[j], None, bias, outs[j], w, None, None, c1["out_mult"], c1["out_shift"],
                                           W, H, Ci, W, H, Co, 1, 1, 0, 0, 0, 0, 1, 1, c1["relu"], c1["bn"])
 
-    wall_ms, dev_ms, repeats = time_launches(step_c1, args.steps, args.warmup)
+    wall_ms, dev_ms, timing = time_launches(step_c1, args.steps, args.warmup)
 
     # parity of what was just computed, on a sample of the batch (the oracle is the checker, outside the timed region)
     import oracle
@@ -172,7 +193,8 @@ def main():
         "config": {"workload": "configs[1]: pointwise 1x1 conv 28x28x128 -> 256, batch 256, "
                                "out_mult/out_shift requantisation + ReLU (pulp_nn_pointwise_HoWo_parallel)",
                    "batch": B, "gemm_MxNxK": [B * H * W, Co, Ci], "buffer_sets_rotated": nset},
-        "timed_regions": repeats,
+        "timed_regions": timing["regions"],
+        "timing": timing,
         "images_per_s": round(B / (wall_ms * 1e-3), 1),
         "device_ms_per_step": round(dev_ms, 5),
         "parity": "bit-exact vs CPU oracle on %d images of every buffer set" % nchk if parity else "MISMATCH vs CPU oracle",
@@ -190,14 +212,15 @@ def main():
             # line for this kernel
             "traffic": traffic_for(traffic, head_kernel),
             "traffic_source": "profiles/bench_all_layers_hbm_traffic.txt",
+            "traffic_measured_in_this_run": False,
         },
     }
 
     # ---- the other single-layer configurations ------------------------------
     layers = []
 
-    def layer_record(name, ops, nbytes, wall, dev, ok, bound, kernel, **extra):
-        rec_ = {"layer": name, "ms": round(dev, 5), "wall_ms": round(wall, 5),
+    def layer_record(name, ops, nbytes, wall, dev, tm, ok, bound, kernel, **extra):
+        rec_ = {"layer": name, "ms": round(dev, 5), "wall_ms": round(wall, 5), "timing": tm["device_us_per_step"],
                 "gops": round(ops / (dev * 1e-3) / 1e9, 1),
                 "mfma_frac": round(ops / (dev * 1e-3) / PEAK_INT8_OPS, 4),
                 "hbm_gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
@@ -227,10 +250,10 @@ def main():
             L.pulp_nn_conv_Ho_parallel(xs0[j], None, b0, outs0[j], w0, k0, l0, 0, c0["out_shift"], 16, 16, 32, 16, 16,
                                        64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
 
-        wall, dev, _ = time_launches(step_c0, steps, warm)
+        wall, dev, tm = time_launches(step_c0, steps, warm)
         want = oracle.conv(c0["x"][:8], c0["w"], c0["bias"], c0["k"], c0["lam"], 0, c0["out_shift"], c0["pads"],
                            c0["strides"], 1, 1, 32)
-        layer_record(c0["name"] + "_b256", c0["ops"], c0["bytes"], wall, dev,
+        layer_record(c0["name"] + "_b256", c0["ops"], c0["bytes"], wall, dev, tm,
                      np.array_equal(outs0[0][:8].cpu().numpy(), want), "mfma",
                      "igemm_kernel<2, 2, 2, 3, 0, 4, 5> (128 x 64 tiles, whole K in one pass)",
                      note="6.3 MB and 2.4 GOP per launch: bound by launch and memory latency, not by a pipe")
@@ -262,8 +285,8 @@ def main():
                 want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
                                                 (1, 1, 1, 1), (2, 2), 1, 1, 32)
                 kern = "dw3x3_lin_kernel<2, 1, 0, true, true>"
-            wall, dev, _ = time_launches(step_c2, steps, warm)
-            layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev,
+            wall, dev, tm = time_launches(step_c2, steps, warm)
+            layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev, tm,
                          np.array_equal(outs2[0][:2].cpu().numpy(), want), "hbm", kern)
             del xs2, outs2
 
@@ -282,15 +305,15 @@ def main():
             L4.pulp_nn_conv_Ho_parallel(xs4[j], None, b4, outs4[j], w4, k4, l4, 0, c4["out_shift"], 64, 64, 256, 63, 63,
                                         256, 3, 3, 1, 0, 1, 0, 1, 1, 1, 1)
 
-        wall, dev, _ = time_launches(step_c4, max(5, steps // 4), 2, min_ms=8.0)
+        wall, dev, tm = time_launches(step_c4, max(5, steps // 4), 2)
         want = oracle.conv(c4["x"][:1], c4["w"], c4["bias"], c4["k"], c4["lam"], 0, c4["out_shift"], c4["pads"],
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
-        layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev,
+        layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev, tm,
                      np.array_equal(outs4[0][:1].cpu().numpy(), want), "mfma",
-                     "igemm_dma_kernel<0> (256 x 256 tiles, LDS-direct loads)",
-                     note="random int8 operands: the matrix cores alone sustain 3.6-4.0 POP/s on this data "
-                          "(clock drops under the power limit), 2.7-3.0 POP/s with the tile's operand feed from "
-                          "LDS: profiles/mfma_ceiling.txt")
+                     "igemm_ring_kernel<0, 4, 0> (persistent workgroups on 256 x 256 tiles, LDS-direct loads)",
+                     note="random int8 operands: the matrix cores alone sustain 3.6-4.0 POP/s on this data (the clock "
+                          "drops under the power limit: profiles/mfma_ceiling.txt); where this kernel's time goes, part "
+                          "by part: profiles/conv_cfg4_phases_ablation.txt")
         # the rest of configuration 4: maxpool 2x2 s2 (63 -> 32) and the 1024 -> 4096 linear layer
         pooled = [torch.zeros((64, 32, 32, 256), dtype=torch.uint8, device="cuda") for _ in range(nset)]
 
@@ -298,10 +321,10 @@ def main():
             j = i % nset
             L4.pulp_nn_maxpool(outs4[j], pooled[j], 63, 63, 256, 32, 32, 2, 2, 0, 0, 0, 0, 2, 2)
 
-        wall, dev, _ = time_launches(step_mp, steps, warm)
+        wall, dev, tm = time_launches(step_mp, steps, warm)
         want = oracle.maxpool(outs4[0][:2].cpu().numpy(), (2, 2), (2, 2), out_hw=(32, 32))
         mp_bytes = 64 * (63 * 63 * 256 + 32 * 32 * 256)
-        layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev,
+        layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev, tm,
                      np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", "maxpool16_kernel<false>")
         gen = torch.Generator(device="cuda")
         gen.manual_seed(20244)
@@ -312,11 +335,11 @@ def main():
         def step_lin(i):
             L4.pulp_nn_linear(vec, lb, lout, lw, lk, ll, 0, c4["lin_shift"], 1024, 4096, 1, 1)
 
-        wall, dev, _ = time_launches(step_lin, steps, warm)
+        wall, dev, tm = time_launches(step_lin, steps, warm)
         want = oracle.linear(vec.cpu().numpy(), c4["lin_w"], c4["lin_bias"], c4["lin_k"], c4["lin_lam"], 0,
                              c4["lin_shift"], 1, 1, 64)
         layer_record("cfg4_linear_1024_4096_b64", 2 * 64 * 1024 * 4096, 64 * (1024 + 4096) + 4096 * 1024 + 4096 * 17,
-                     wall, dev, np.array_equal(lout.cpu().numpy(), want), "hbm", "linear_skinny_kernel<0>",
+                     wall, dev, tm, np.array_equal(lout.cpu().numpy(), want), "hbm", "linear_skinny_kernel<0>",
                      note="4.5 MB per launch: bound by launch and memory latency")
         del xs4, outs4, pooled
 
@@ -330,7 +353,7 @@ def main():
         def step_net(i):
             runner.run(x3)
 
-        wall, dev, _ = time_launches(step_net, max(5, steps // 4), 2, min_ms=8.0)
+        wall, dev, tm = time_launches(step_net, max(5, steps // 4), 2)
         libs[32].sync()
         import hashlib
         dig = json.load(open(os.path.join(ROOT, "tests", "golden", "config_digests.json")))["cfg3_b256_logits"]["sha256"]
@@ -338,7 +361,7 @@ def main():
         if not ok:
             failures.append("cfg3 chain")
         layers.append({"layer": "cfg3_mobilenet_v1_0.5_128x128_b256 (whole chain)", "ms": round(dev, 5),
-                       "wall_ms": round(wall, 5), "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
+                       "wall_ms": round(wall, 5), "timing": tm["device_us_per_step"], "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
                        "launches": runner.launches if hasattr(runner, "launches") else None,
                        "images_per_s": round(256 / (wall * 1e-3), 1),
                        "mfma_frac": round(net["ops"] / (dev * 1e-3) / PEAK_INT8_OPS, 4),
@@ -407,6 +430,45 @@ def main():
             "sample": "%d x %d images of the same workload (scalar C restatement of the reference, -O3 "
                       "-march=native, one image row per OpenMP task), %.1f s" % (reps, n_img, el),
             "images_per_s": round(n_img * reps / el, 1)}
+
+        # configs[0] as BASELINE.json states it: batch 1, one thread (the reference runs one image on one cluster)
+        def cpu_timed(fn, budget_s):
+            fn()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                fn()
+                reps += 1
+                el = time.perf_counter() - t0
+                if el > budget_s:
+                    return el / reps, reps
+
+        c0 = workloads.config0(batch=1)
+        sec, reps = cpu_timed(lambda: oracle.conv(c0["x"], c0["w"], c0["bias"], c0["k"], c0["lam"], 0, c0["out_shift"],
+                                                  c0["pads"], c0["strides"], 1, 1, 32, nthreads=1), 2.0)
+        rec["cpu_baseline_cfg0_b1"] = {
+            "value": round(c0["ops"] / sec / 1e9, 2), "unit": "GOPS", "cores": 1, "kind": "port",
+            "ms_per_image": round(sec * 1e3, 4), "images_per_s": round(1.0 / sec, 1),
+            "sample": "configs[0] (3x3 conv 16x16x32 -> 64, 32-bit batch-norm + ReLU), batch 1, one thread, %d runs" % reps}
+        if not args.no_layers:
+            # the other layers on the host cores, a few images each (reported baselines, not targets)
+            cpu_layers = {}
+            c2 = workloads.config2(batch=2 * threads, stride=1)
+            xin = np.pad(c2["x"], ((0, 0), (0, 0), (1, 1), (0, 0)))
+            sec, reps = cpu_timed(lambda: oracle.depthwise_3x3_s1(xin, c2["w"], c2["k"], c2["lam"], 0, c2["out_shift"], 1, 1,
+                                                                 1, 1, 32, nthreads=threads), 3.0)
+            cpu_layers["cfg2_depthwise3x3_s1"] = {"gops": round(c2["ops"] / sec / 1e9, 2), "images_per_s": round(2 * threads / sec, 1)}
+            c2 = workloads.config2(batch=2 * threads, stride=2)
+            sec, reps = cpu_timed(lambda: oracle.depthwise_generic(c2["x"], c2["w"], c2["bias"], c2["k"], c2["lam"], 0,
+                                                                  c2["out_shift"], (1, 1, 1, 1), (2, 2), 1, 1, 32,
+                                                                  nthreads=threads), 3.0)
+            cpu_layers["cfg2_depthwise3x3_s2"] = {"gops": round(c2["ops"] / sec / 1e9, 2), "images_per_s": round(2 * threads / sec, 1)}
+            c4 = workloads.config4(batch=1, relu=1)
+            sec, reps = cpu_timed(lambda: oracle.conv(c4["x"], c4["w"], c4["bias"], c4["k"], c4["lam"], 0, c4["out_shift"],
+                                                      c4["pads"], c4["strides"], 1, 1, 64, out_hw=(63, 63), nthreads=threads), 5.0)
+            cpu_layers["cfg4_conv3x3_bn64"] = {"gops": round(c4["ops"] / sec / 1e9, 2), "images_per_s": round(1.0 / sec, 2)}
+            rec["cpu_baseline_layers"] = {"cores": threads, "kind": "port", "layers": cpu_layers,
+                                          "sample": "2 x cores images per depthwise call, one image per convolution call, "
+                                                    "3-5 s each"}
 
     if failures:
         rec["value"] = None
