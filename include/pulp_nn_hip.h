@@ -117,7 +117,7 @@ typedef struct pulp_nn_hip_block {
  * The result is bit for bit that of n_blocks calls of pulp_nn_hip_dw_pw_hwc.  Supported: what
  * pulp_nn_hip_dw_pw_hwc supports at stride 1 with ch_out == ch, images small enough for a
  * workgroup to hold whole ones (dim_im_x x dim_im_y x ch x 2 bytes and the constants within 64 KB
- * of LDS: 8 x 8 x 256, 16 x 16 x 64, 4 x 4 x 1024 ...), and a batch that is a multiple of the
+ * of LDS: 8 x 8 x 256, 16 x 16 x 64, 4 x 4 x 512 ...), and a batch that is a multiple of the
  * images a workgroup takes.  Anything else sets PULP_NN_HIP_ERR_UNSUPPORTED and queues nothing:
  * call pulp_nn_hip_dw_pw_hwc per block instead. */
 void pulp_nn_hip_dw_pw_chain_hwc(const unsigned char *Im_in, unsigned char *Im_out, unsigned short dim_im_x,

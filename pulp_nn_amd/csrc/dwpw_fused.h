@@ -34,6 +34,7 @@
 #include "igemm.h"
 
 #define DWPW_MAX_BLOCKS 8  // blocks of one launch (pulp_nn_hip_dw_pw_chain_hwc)
+#define DWPW_YPAD 64        // padding bytes per pixel of a block's output kept in LDS for the next block
 
 // one depthwise + pointwise block
 struct DwPwBlock {
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
   const int nch = max(nb_hi - nb_lo, 0) * 64;
   int *c_bias = (int *)(dwpw_lds + dwpw_lds_bytes(g.BM, g.C));
   bn_t *c_k = (bn_t *)(c_bias + nch), *c_l = c_k + nch;
-  // the output of a block that another block follows: [tile pixel][Co] bytes, the next block's HWC input
+  // the output of a block that another block follows: [tile pixel][Co + DWPW_YPAD] bytes, the next block's HWC input
   unsigned char *ylds = dwpw_lds + dwpw_lds_bytes(g.BM, g.C) + dwpw_const_bytes(nch);
   typedef unsigned v4u __attribute__((ext_vector_type(4)));
   const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
@@ -179,17 +180,20 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
         unsigned row[NIN][RD];
         // the image this item lies in: in memory for the first block, else where the block before left it (a tile of
         // several blocks is made of whole images, stride 1: image (b - first image of the tile) of the tile)
+        // (in LDS a pixel takes 64 bytes more than its channels: with the power-of-two pitch the four pixels a lane
+        // quad reads here, and the pixels a store of the epilogue writes, would all start in the same bank)
+        const int pitch = first ? g.C : g.C + DWPW_YPAD;
         const uint8_t *img = first ? g.in + (long long)b * g.H * WB * g.C
-                                   : ylds + (long long)(b - (int)fastdiv((unsigned)m0, g.d_howo)) * g.H * WB * g.C;
-        const uint8_t *src = img + (lane & 3) * g.C + (ch & ~3);
+                                   : ylds + (long long)(b - (int)fastdiv((unsigned)m0, g.d_howo)) * g.H * WB * pitch;
+        const uint8_t *src = img + (lane & 3) * pitch + (ch & ~3);
 #pragma unroll
         for (int r = 0; r < NIN; r++) {
           const int iy = oy0 * S - 1 + r;
           const bool ok = (unsigned)iy < (unsigned)g.H;
-          const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB * g.C;
+          const uint8_t *rp = src + (long long)min(max(iy, 0), g.H - 1) * WB * pitch;
 #pragma unroll
           for (int d = 0; d < RD; d++) {
-            const unsigned v = *(const unsigned *)(rp + (long long)(4 * d) * g.C);
+            const unsigned v = *(const unsigned *)(rp + (long long)(4 * d) * pitch);
             row[r][d] = ok ? v : 0u;
           }
         }
@@ -346,7 +350,7 @@ __global__ __launch_bounds__(64 * NWV) void dwpw_fused_kernel(DwPwGeom g)
         if (m0 + pl < g.M && cb < g.Co) {
           const v4i v = {(int)packed[s][0], (int)packed[s][1], (int)packed[s][2], (int)packed[s][3]};
           if (last) *(v4i *)(g.out + (long long)(m0 + pl) * g.Co + cb) = v;
-          else *(v4i *)(ylds + pl * g.Co + cb) = v;
+          else *(v4i *)(ylds + pl * (g.Co + DWPW_YPAD) + cb) = v;
         }
       }
     }

@@ -25,6 +25,7 @@
 #include "dwpw_fused.h"
 #include "igemm.h"
 #include "igemm_ring.h"
+#include "depthwise_stream.h"
 #include "linear_skinny.h"
 #include "pool.h"
 #include "pw_stream.h"
@@ -248,6 +249,12 @@ void launch_smallk(int mode, bool rows, ConvGeom &g, const EpiArgs &e, hipStream
   g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
   dim3 grid((unsigned)((g.M + 255) / 256)), block(256);
   if (rows) {
+    // runs of 256 pixels per workgroup: as many as leave every compute unit its eight workgroups
+    const long long runs = (g.M + 255) / 256;
+    g.tiles_n = (int)std::max<long long>(1, std::min<long long>(8, runs / (8ll * num_cus())));
+    g.d_howo = fastdiv_make((unsigned)g.HoWo);
+    g.d_wo = fastdiv_make((unsigned)g.Wo);
+    grid = dim3((unsigned)((runs + g.tiles_n - 1) / g.tiles_n));
     switch (mode) {
       case EPI_BN: hipLaunchKernelGGL((smallk_rows_kernel<NCH, EPI_BN>), grid, block, 0, s, g, e); break;
       case EPI_MULT: hipLaunchKernelGGL((smallk_rows_kernel<NCH, EPI_MULT>), grid, block, 0, s, g, e); break;
@@ -574,6 +581,12 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
   const bool rowsk = !plane && fast && pt == 1 && pl == 1 && (W == 16 || W == 32 || W == 64) && Wo == (W - 1) / sx + 1 &&
                      Ho <= (H - 1) / sy + 1 && CH % 4 == 0 && ((long long)g_batch * CH) % DW_CG == 0 && aligned(in, hwc_in ? 4 : 16) &&
                      aligned(out, 4) && (long long)g_batch * CH / DW_CG * Ho < 0x7fffffffLL;
+  // Layers that fill the machine with one workgroup per image and 64 channels (two per compute unit): the plane
+  // streamed through LDS, 8 rows of it per request.  Up to 14 groups of 4 output columns, 64 KiB of LDS.
+  const int stream_csd = (2 * DWS_ROWS * (W / 4)) | 1;
+  const size_t stream_lds = 4 * ((size_t)DW_CG * stream_csd + 8 * (size_t)(Wo / 4));
+  const bool stream = !plane && !rowsk && !hwc_in && lin_dma_ok && Wo / 4 <= 16 - DWS_LOADERS && stream_lds <= 64 * 1024 &&
+                      (long long)g_batch * (CH / DW_CG) >= 2ll * num_cus();
   if (hwc_in && !plane && !rowsk)
     return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "no fused kernel for this geometry: use pulp_nn_hip_hwc_to_chw and the CHW entry point");
   if (plane) {
@@ -618,6 +631,25 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
     else DWR_MODE(64, 2, 2)
 #undef DWR_MODE
 #undef DWR_LAYOUT
+  } else if (stream) {
+    // whole planes streamed through LDS by loader waves, one workgroup per image and 64 channels
+    g.NR = DWS_ROWS;
+    g.RB = 2;
+    g.CSD = stream_csd;
+    g.bands = 1;
+    g.total = (int)((long long)g.B * g.cgroups);
+    const dim3 sgrid(g.total), sblock(64 * (Wo / 4 + DWS_LOADERS));
+#define DWS_MODE(S, PL)                                                                                                  \
+  switch (mode) {                                                                                                        \
+    case EPI_BN: hipLaunchKernelGGL((dw3x3_stream_kernel<S, PL, EPI_BN>), sgrid, sblock, stream_lds, g_stream, g, e); break;     \
+    case EPI_MULT: hipLaunchKernelGGL((dw3x3_stream_kernel<S, PL, EPI_MULT>), sgrid, sblock, stream_lds, g_stream, g, e); break; \
+    default: hipLaunchKernelGGL((dw3x3_stream_kernel<S, PL, EPI_RAW>), sgrid, sblock, stream_lds, g_stream, g, e); break;        \
+  }
+    if (sx == 1 && pl == 1) { DWS_MODE(1, 1) }
+    else if (sx == 1) { DWS_MODE(1, 0) }
+    else if (pl == 1) { DWS_MODE(2, 1) }
+    else { DWS_MODE(2, 0) }
+#undef DWS_MODE
   } else if (lin) {
     const bool full = (Wo % 4 == 0) && (g.CH % DW_CG == 0) && (g.planes % DW_CG == 0) && g.out_vec4;
     const size_t ldsl = lds + 16;  // spare dword for masked-off staging writes
@@ -1133,7 +1165,7 @@ static void dwpw_common(const char *fn, const unsigned char *Im_in, unsigned cha
     g.BM = per_tile * img_px;
     tiles = (int)((M + g.BM - 1) / g.BM);
     g.nsplit = 1;
-    lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(nbt * 64) + (size_t)g.BM * Co;
+    lds = (size_t)dwpw_lds_bytes(g.BM, C) + (size_t)dwpw_const_bytes(nbt * 64) + (size_t)g.BM * (Co + DWPW_YPAD);
     if (S != 1 || C != Co || g_batch % (unsigned)per_tile != 0)
       return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "blocks can only be chained at stride 1 with as many channels out as in, on whole images per tile");
   }

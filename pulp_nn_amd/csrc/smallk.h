@@ -177,97 +177,126 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
   }
   __syncthreads();
 
-  // ---- this lane's pixel: its (up to) three filter rows ------------------------------------
-  const int m = blockIdx.x * 256 + tid;
-  if (m >= g.M) return;
-  const int b = m / g.HoWo, rem = m - b * g.HoWo;
-  const int oy = rem / g.Wo, ox = rem - oy * g.Wo;
-  const int iy0 = oy * g.sy - g.pt, ix0 = ox * g.sx - g.pl;
+  // ---- this lane's pixels: the (up to) three filter rows of each ---------------------------------
+  // A workgroup takes g.tiles_n runs of 256 consecutive pixels (the weight table and the two barriers above are
+  // set up once for all of them, not once per 256 pixels); the rows of the next run's pixel are requested before
+  // this run's pixel is multiplied.
   const unsigned batch = (unsigned)((g.M + g.HoWo - 1) / g.HoWo);
   const int total = (int)(batch * (unsigned)g.in_img);  // bytes of input
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)g.in, 0, total, 0x00020000);
-  // bytes [lo, hi) of a filter row lie inside the image
-  const int lo = max(0, -ix0) * g.Ci, hi = max(min(g.kx, g.W - ix0), 0) * g.Ci;
-  const unsigned bits = ((1u << hi) - 1u) & ~((1u << lo) - 1u);  // hi <= 12
-  unsigned md[SMALLK_RD];
-#pragma unroll
-  for (int i = 0; i < SMALLK_RD; i++) md[i] = ((((bits >> (4 * i)) & 15u) * 0x00204081u) & 0x01010101u) * 0xFFu;
-  const int rowpos = (int)((unsigned)b * (unsigned)g.in_img) + ix0 * g.Ci;  // byte offset of the row's first byte, less iy * W * Ci
   typedef unsigned v3u __attribute__((ext_vector_type(3)));
-  unsigned a[3][SMALLK_RD];
+  struct Rows {
+    v3u d[3];              // the 12 bytes from the aligned address below each row's first byte
+    int sh[3];             // where the row starts in them
+    unsigned md[SMALLK_RD];  // byte mask of the columns inside the image
+    int A0, lo, hi, iy0;   // (for the few lanes whose load would leave the input: see finish())
+    bool ok[3];
+  };
+  auto request = [&](int m, Rows &R) {
+    const bool live = m < g.M;
+    const int mm = live ? m : 0;
+    const int b = (int)fastdiv((unsigned)mm, g.d_howo), rem = mm - b * g.HoWo;
+    const int oy = (int)fastdiv((unsigned)rem, g.d_wo), ox = rem - oy * g.Wo;
+    const int iy0 = oy * g.sy - g.pt, ix0 = ox * g.sx - g.pl;
+    // bytes [lo, hi) of a filter row lie inside the image
+    const int lo = max(0, -ix0) * g.Ci, hi = max(min(g.kx, g.W - ix0), 0) * g.Ci;
+    const unsigned bits = ((1u << hi) - 1u) & ~((1u << lo) - 1u);  // hi <= 12
 #pragma unroll
-  for (int fy = 0; fy < 3; fy++) {
-    const int iy = iy0 + fy;
-    const bool ok = fy < g.ky && (unsigned)iy < (unsigned)g.H;
-    const int A = rowpos + iy * g.W * g.Ci;
-    const int sh = A & 3, base = A - sh;
-    // The 12 bytes from the aligned address below the row's first byte, as one range-checked
-    // load; a row outside the image is given an offset that is out of range, which loads zeros.
-    const v3u d = __builtin_amdgcn_raw_buffer_load_b96(rsrc, ok ? base : (int)0xfffffff0, 0, 0);
-    unsigned r0 = __builtin_amdgcn_alignbyte(d.y, d.x, sh);
-    unsigned r1 = __builtin_amdgcn_alignbyte(d.z, d.y, sh);
-    unsigned r2 = __builtin_amdgcn_alignbyte(0u, d.z, sh);
-    // The load must lie inside the input as a whole.  Where it would not (left padding in the
-    // first row of the first image, the last bytes of the last image), the few lanes concerned
-    // fetch the bytes of the row that lie inside the image one by one.
-    if (ok && (base < 0 || base + 12 > total)) {
-      unsigned t[SMALLK_RD] = {0, 0, 0};
+    for (int i = 0; i < SMALLK_RD; i++) R.md[i] = ((((bits >> (4 * i)) & 15u) * 0x00204081u) & 0x01010101u) * 0xFFu;
+    const int rowpos = (int)((unsigned)b * (unsigned)g.in_img) + ix0 * g.Ci;  // byte offset of the row's first byte, less iy * W * Ci
+    R.A0 = rowpos, R.lo = lo, R.hi = hi, R.iy0 = iy0;
 #pragma unroll
-      for (int j = 0; j < 4 * SMALLK_RD; j++)
-        if (j >= lo && j < hi) t[j >> 2] |= (unsigned)g.in[A + j] << (8 * (j & 3));
-      r0 = t[0];
-      r1 = t[1];
-      r2 = t[2];
+    for (int fy = 0; fy < 3; fy++) {
+      const int iy = iy0 + fy;
+      R.ok[fy] = live && fy < g.ky && (unsigned)iy < (unsigned)g.H;
+      const int A = rowpos + iy * g.W * g.Ci;
+      R.sh[fy] = A & 3;
+      // one range-checked load; a row outside the image is given an offset that is out of range, which loads zeros
+      R.d[fy] = __builtin_amdgcn_raw_buffer_load_b96(rsrc, R.ok[fy] ? A - R.sh[fy] : (int)0xfffffff0, 0, 0);
     }
-    a[fy][0] = (r0 & md[0]) ^ 0x80808080u;
-    a[fy][1] = (r1 & md[1]) ^ 0x80808080u;
-    a[fy][2] = (r2 & md[2]) ^ 0x80808080u;
-  }
+  };
+  auto finish = [&](const Rows &R, unsigned (&a)[3][SMALLK_RD]) {
+#pragma unroll
+    for (int fy = 0; fy < 3; fy++) {
+      unsigned r0 = __builtin_amdgcn_alignbyte(R.d[fy].y, R.d[fy].x, R.sh[fy]);
+      unsigned r1 = __builtin_amdgcn_alignbyte(R.d[fy].z, R.d[fy].y, R.sh[fy]);
+      unsigned r2 = __builtin_amdgcn_alignbyte(0u, R.d[fy].z, R.sh[fy]);
+      // The load must lie inside the input as a whole.  Where it would not (left padding in the
+      // first row of the first image, the last bytes of the last image), the few lanes concerned
+      // fetch the bytes of the row that lie inside the image one by one.
+      const int A = R.A0 + (R.iy0 + fy) * g.W * g.Ci, base = A - R.sh[fy];
+      if (R.ok[fy] && (base < 0 || base + 12 > total)) {
+        unsigned t[SMALLK_RD] = {0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4 * SMALLK_RD; j++)
+          if (j >= R.lo && j < R.hi) t[j >> 2] |= (unsigned)g.in[A + j] << (8 * (j & 3));
+        r0 = t[0];
+        r1 = t[1];
+        r2 = t[2];
+      }
+      a[fy][0] = (r0 & R.md[0]) ^ 0x80808080u;
+      a[fy][1] = (r1 & R.md[1]) ^ 0x80808080u;
+      a[fy][2] = (r2 & R.md[2]) ^ 0x80808080u;
+    }
+  };
+  const int npass = g.tiles_n;
+  int m = blockIdx.x * npass * 256 + tid;
+  Rows cur, nxt;
+  request(m, cur);
+#pragma unroll 1
+  for (int pass = 0; pass < npass; pass++, m += 256) {
+    if (pass + 1 < npass) request(m + 256, nxt);
+    unsigned a[3][SMALLK_RD];
+    finish(cur, a);
 
-  // ---- NCH dot products, requantise, store ----------------------------------------------
-  unsigned packed[NCH / 4];
+    // ---- NCH dot products, requantise, store ----------------------------------------------
+    unsigned packed[NCH / 4];
 #pragma unroll
-  for (int n4 = 0; n4 < NCH / 4; n4++) {
-    int acc[4];
+    for (int n4 = 0; n4 < NCH / 4; n4++) {
+      int acc[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int n = 4 * n4 + r;
-      acc[r] = corr_l[n];
-      const v4i w0 = *(const v4i *)&wl[n * SMALLK_RP], w1 = *(const v4i *)&wl[n * SMALLK_RP + 4];
-      const int w2 = wl[n * SMALLK_RP + 8];
-      acc[r] = __builtin_amdgcn_sdot4((int)a[0][0], w0.x, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[0][1], w0.y, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[0][2], w0.z, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[1][0], w0.w, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[1][1], w1.x, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[1][2], w1.y, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[2][0], w1.z, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[2][1], w1.w, acc[r], false);
-      acc[r] = __builtin_amdgcn_sdot4((int)a[2][2], w2, acc[r], false);
+      for (int r = 0; r < 4; r++) {
+        const int n = 4 * n4 + r;
+        acc[r] = corr_l[n];
+        const v4i w0 = *(const v4i *)&wl[n * SMALLK_RP], w1 = *(const v4i *)&wl[n * SMALLK_RP + 4];
+        const int w2 = wl[n * SMALLK_RP + 8];
+        acc[r] = __builtin_amdgcn_sdot4((int)a[0][0], w0.x, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[0][1], w0.y, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[0][2], w0.z, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[1][0], w0.w, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[1][1], w1.x, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[1][2], w1.y, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[2][0], w1.z, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[2][1], w1.w, acc[r], false);
+        acc[r] = __builtin_amdgcn_sdot4((int)a[2][2], w2, acc[r], false);
+      }
+      unsigned p = 0;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int n = 4 * n4 + r;
+        const bn_t kk = (MODE == EPI_BN) ? k_l[n] : (bn_t)0, ll = (MODE == EPI_BN) ? lam_l[n] : (bn_t)0;
+        p |= (unsigned)requant<MODE>(acc[r], kk, ll, e.mult, e.shift) << (8 * r);
+      }
+      packed[n4] = p;
     }
-    unsigned p = 0;
+    if (m < g.M) {
+      uint8_t *o = (uint8_t *)g.out + (long long)m * g.N;
+      if (g.vec_store) {
+        // N == NCH and 16-byte aligned rows: one copy of the store code per cache policy
+        auto put = [&](auto nt) {
+          constexpr bool NT = decltype(nt)::value;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int n = 4 * n4 + r;
-      const bn_t kk = (MODE == EPI_BN) ? k_l[n] : (bn_t)0, ll = (MODE == EPI_BN) ? lam_l[n] : (bn_t)0;
-      p |= (unsigned)requant<MODE>(acc[r], kk, ll, e.mult, e.shift) << (8 * r);
+          for (int q = 0; q < NCH / 16; q++)
+            store16<NT>(o + 16 * q, (v4i){(int)packed[4 * q], (int)packed[4 * q + 1], (int)packed[4 * q + 2], (int)packed[4 * q + 3]});
+        };
+        if (g.nt) put(std::true_type{});
+        else put(std::false_type{});
+      } else {
+#pragma unroll
+        for (int n = 0; n < NCH; n++)
+          if (n < g.N) o[n] = (uint8_t)(packed[n >> 2] >> (8 * (n & 3)));
+      }
     }
-    packed[n4] = p;
-  }
-  uint8_t *o = (uint8_t *)g.out + (long long)m * g.N;
-  if (g.vec_store) {
-    // N == NCH and 16-byte aligned rows: one copy of the store code per cache policy
-    auto put = [&](auto nt) {
-      constexpr bool NT = decltype(nt)::value;
-#pragma unroll
-      for (int q = 0; q < NCH / 16; q++)
-        store16<NT>(o + 16 * q, (v4i){(int)packed[4 * q], (int)packed[4 * q + 1], (int)packed[4 * q + 2], (int)packed[4 * q + 3]});
-    };
-    if (g.nt) put(std::true_type{});
-    else put(std::false_type{});
-  } else {
-#pragma unroll
-    for (int n = 0; n < NCH; n++)
-      if (n < g.N) o[n] = (uint8_t)(packed[n >> 2] >> (8 * (n & 3)));
+    cur = nxt;
   }
 }
