@@ -38,7 +38,7 @@ def build(bn_bits, verbose=False):
     return out
 
 
-TOOLS = ("mfma_ceiling", "conv_phases")
+TOOLS = ("mfma_ceiling", "conv_phases", "hbm_ceiling")
 
 
 def tool_path(name="mfma_ceiling"):
@@ -47,7 +47,7 @@ def tool_path(name="mfma_ceiling"):
 
 def build_tool(name="mfma_ceiling", verbose=False):
     """The measurement tools: the matrix-core yardstick (csrc/mfma_ceiling.hip) and the phase / ablation trace of
-    the large convolution (csrc/conv_phases.hip).  Stand-alone executables, no part of the libraries."""
+    the large convolution (csrc/conv_phases.hip), the plain-copy memory yardstick (csrc/hbm_ceiling.hip).  Stand-alone executables, no part of the libraries."""
     os.makedirs(LIBDIR, exist_ok=True)
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
            "-packed-fp32-ops", os.path.join(CSRC, name + ".hip"), "-o", tool_path(name)]

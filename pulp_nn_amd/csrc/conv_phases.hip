@@ -24,6 +24,7 @@
 
 #include "igemm.h"
 #include "igemm_ring.h"
+#include "igemm_patch.h"
 
 #define CK(x)                                                              \
   do {                                                                     \
@@ -47,9 +48,26 @@ static int g_cus = 256;
 static const int B = 64, H = 64, W = 64, Ci = 256, Co = 256, Ho = 63, Wo = 63;
 static const double OPS = 2.0 * B * Ho * Wo * Co * 9 * Ci;
 
+// WN = 0: igemm_patch_kernel (4 x 64 pixel patches, an input row staged once per filter row)
 template <int WN, int ABL>
 static int launch(ConvGeom g, EpiArgs e)
 {
+  if constexpr (WN == 0) {
+    g.tiles_n = (g.N + IGP_BN - 1) / IGP_BN;
+    g.rgroups = (g.Ho + 3) / 4;
+    g.d_rg = fastdiv_make(g.rgroups);
+    g.tiles_total = g.batch * g.rgroups * g.tiles_n;
+    g.d_tiles_n = fastdiv_make(g.tiles_n);
+    const int unit = 8 * g.tiles_n;
+    const int grid = g_cus / unit * unit;
+    static bool raised = false;
+    if (!raised) {
+      CK(hipFuncSetAttribute((const void *)igemm_patch_kernel<EPI_BN, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, igp_lds_bytes()));
+      raised = true;
+    }
+    hipLaunchKernelGGL((igemm_patch_kernel<EPI_BN, ABL>), dim3(grid), dim3(IGP_THREADS), igp_lds_bytes(), 0, g, e);
+    return grid;
+  } else {
   typedef IgrShape<WN> S;
   g.tiles_n = (g.N + S::BN - 1) / S::BN;
   g.tiles_total = ((g.M + IGR_BM - 1) / IGR_BM) * g.tiles_n;
@@ -63,6 +81,7 @@ static int launch(ConvGeom g, EpiArgs e)
   }
   hipLaunchKernelGGL((igemm_ring_kernel<EPI_BN, WN, ABL>), dim3(grid), dim3(S::THREADS), S::lds_bytes(), 0, g, e);
   return grid;
+  }
 }
 
 template <int WN, int ABL>
@@ -166,7 +185,39 @@ int main()
          prop.gcnArchName, g_cus, OPS / 1e9);
   printf("columns: settled launch-to-launch time (median of the second half of 2000 launches back to back) | mean of the first 50 launches |\n"
          "         rounds 1 and 2 of a traced launch, mean over the workgroups | shader cycles per wall-clock time over the main loop\n");
-  printf("-- one workgroup of eight waves per compute unit, 256 x 256 tiles (the library's kernel) --\n");
+  {
+    // the two kernels against each other, byte by byte
+    std::vector<uint8_t> a(nout), b(nout);
+    CK(hipMemset(dout, 0xA5, nout));
+    launch<4, 0>(g, e);
+    CK(hipDeviceSynchronize());
+    CK(hipMemcpy(a.data(), dout, nout, hipMemcpyDeviceToHost));
+    CK(hipMemset(dout, 0x5A, nout));
+    launch<0, 0>(g, e);
+    CK(hipDeviceSynchronize());
+    CK(hipGetLastError());
+    CK(hipMemcpy(b.data(), dout, nout, hipMemcpyDeviceToHost));
+    size_t bad = 0, fb = 0;
+    for (size_t i = 0; i < nout; i++)
+      if (a[i] != b[i]) {
+        if (!bad) fb = i;
+        bad++;
+      }
+    printf("igemm_patch_kernel against igemm_ring_kernel: %zu of %zu output bytes differ", bad, nout);
+    if (bad) printf(" (first: pixel %zu channel %zu, %d against %d)", fb / Co, fb % Co, b[fb], a[fb]);
+    printf("\n");
+    fflush(stdout);
+    if (bad) return 1;
+  }
+  printf("-- 4 x 64 pixel patches, input rows staged once per filter row (igemm_patch_kernel; the library's kernel for this layer) --\n");
+  run<0, 0>("complete", g, e, dtr, true);
+  run<0, 1>("no loads behind a tile's first two groups", g, e, dtr, false);
+  run<0, 4>("no fragment reads in the loop", g, e, dtr, false);
+  run<0, 8>("no epilogue", g, e, dtr, false);
+  run<0, 32>("activation loads out of range (zeros, no traffic)", g, e, dtr, false);
+  run<0, 64>("weight loads out of range", g, e, dtr, false);
+  run<0, 96>("all loads out of range", g, e, dtr, false);
+  printf("-- 256 consecutive pixels x 256 channels, one sub-slice per tap (igemm_ring_kernel) --\n");
   run<4, 0>("complete", g, e, dtr, true);
   run<4, 1>("no loads behind a tile's first sub-slices", g, e, dtr, false);
   run<4, 4>("no fragment reads in the loop", g, e, dtr, false);

@@ -87,6 +87,8 @@ struct ConvGeom {
   int rkx;             // 65536 / kx + 1: t * rkx >> 16 == t / kx for t < 32 (GATHER_SUBTAP)
   int cpt;             // Ci / 64: K sub-slices per filter tap (igemm_ring_kernel)
   FastDiv d_cpt, d_kx; // divisions by cpt and kx (igemm_ring_kernel)
+  int rgroups;         // groups of 4 output rows per image (igemm_patch_kernel)
+  FastDiv d_rg;        // division by rgroups
 };
 
 #define IGEMM_BK 64

@@ -69,6 +69,54 @@ __device__ long long *igr_trace = nullptr;
 #define IGR_STAMP(i)
 #endif
 
+// Requantisation of four accumulators (consecutive channels of one pixel) with the folded per-channel constants:
+// ll = k * corr + lambda (batch-norm branch), mult * corr (scalar multiplier) or corr (shift only), see the
+// kernels' channel tables.  FORM (batch-norm branch, 64-bit build): 0 = multipliers fit 32 bits and shift >= 32
+// (the result is the high dword of k * acc + l, shifted), 1 = multipliers fit 32 bits (funnel shift of the two
+// dwords), 2 = general 64-bit arithmetic.  Other branches and the 32-bit build have one form.
+template <int MODE, int FORM>
+__device__ __forceinline__ unsigned igr_requant4(const v4i &a, const bn_t (&kk)[4], const bn_t (&ll)[4], const EpiArgs &e)
+{
+  int x[4];
+  if constexpr (MODE == EPI_BN) {
+#if PULPNN_BN_BITS == 64
+    if constexpr (FORM == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) x[r] = (int)(((long long)(int)kk[r] * (long long)a[r] + ll[r]) >> 32);
+      return ashr_sat_pack4(x[0], x[1], x[2], x[3], e.shift - 32);
+    } else if constexpr (FORM == 1) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const long long v = (long long)(int)kk[r] * (long long)a[r] + ll[r];
+        x[r] = (int)__builtin_amdgcn_alignbit((unsigned)(v >> 32), (unsigned)v, e.shift);
+      }
+      return ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
+    } else {
+      unsigned p = 0;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const unsigned long long v = (unsigned long long)kk[r] * (unsigned long long)(long long)a[r] + (unsigned long long)ll[r];
+        p |= (unsigned)clipu8((int)(unsigned)(unsigned long long)((long long)v >> e.shift)) << (8 * r);
+      }
+      return p;
+    }
+#else
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (int)((unsigned)kk[r] * (unsigned)a[r] + (unsigned)ll[r]);
+    return ashr_sat_pack4(x[0], x[1], x[2], x[3], e.shift);
+#endif
+  } else if constexpr (MODE == EPI_MULT) {
+    // (int16_t)((mult * (acc + corr)) >> shift), then clamp
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (int)(short)((int)((unsigned)e.mult * (unsigned)a[r] + (unsigned)ll[r]) >> e.shift);
+    return ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[r] = (a[r] + (int)ll[r]) >> e.shift;
+    return ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
+  }
+}
+
 // ABL (tools only, wrong results): 1 = no loads after a tile's first sub-slices, 2 = one MFMA per
 // sub-slice instead of 32, 4 = no fragment reads in the loop, 8 = no epilogue, 16 = epilogue without its stores.
 template <int MODE, int WN, int ABL = 0>
@@ -369,9 +417,7 @@ __global__ __launch_bounds__(IgrShape<WN>::THREADS, WN == 2 ? 2 : 1) void igemm_
     if (!(ABL & 8) || g.M < 0) {
       const int cb = wave_n * WNC + lgrp * 16;
       unsigned packed[TM][TN];
-      // FORM (batch-norm branch, 64-bit build): 0 = multipliers fit 32 bits and shift >= 32 (the result is the
-      // high dword of k * acc + l, shifted), 1 = multipliers fit 32 bits (funnel shift of the two dwords),
-      // 2 = general 64-bit arithmetic.  Other branches and the 32-bit build have one form.
+      // FORM: see igr_requant4
       auto requantise = [&](auto form_tag) {
         constexpr int FORM = decltype(form_tag)::value;
 #pragma unroll
@@ -383,48 +429,7 @@ __global__ __launch_bounds__(IgrShape<WN>::THREADS, WN == 2 ? 2 : 1) void igemm_
             kk[r] = MODE == EPI_BN ? cmul[cb + 4 * t + r] : (bn_t)0;
           }
 #pragma unroll
-          for (int s = 0; s < TM; s++) {
-            int x[4];
-            if constexpr (MODE == EPI_BN) {
-#if PULPNN_BN_BITS == 64
-              if constexpr (FORM == 0) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) x[r] = (int)(((long long)(int)kk[r] * (long long)acc[t][s][r] + ll[r]) >> 32);
-                packed[s][t] = ashr_sat_pack4(x[0], x[1], x[2], x[3], e.shift - 32);
-              } else if constexpr (FORM == 1) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                  const long long v = (long long)(int)kk[r] * (long long)acc[t][s][r] + ll[r];
-                  x[r] = (int)__builtin_amdgcn_alignbit((unsigned)(v >> 32), (unsigned)v, e.shift);
-                }
-                packed[s][t] = ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
-              } else {
-                unsigned p = 0;
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                  const unsigned long long v =
-                      (unsigned long long)kk[r] * (unsigned long long)(long long)acc[t][s][r] + (unsigned long long)ll[r];
-                  p |= (unsigned)clipu8((int)(unsigned)(unsigned long long)((long long)v >> e.shift)) << (8 * r);
-                }
-                packed[s][t] = p;
-              }
-#else
-#pragma unroll
-              for (int r = 0; r < 4; r++) x[r] = (int)((unsigned)kk[r] * (unsigned)acc[t][s][r] + (unsigned)ll[r]);
-              packed[s][t] = ashr_sat_pack4(x[0], x[1], x[2], x[3], e.shift);
-#endif
-            } else if constexpr (MODE == EPI_MULT) {
-              // (int16_t)((mult * (acc + corr)) >> shift), then clamp
-#pragma unroll
-              for (int r = 0; r < 4; r++)
-                x[r] = (int)(short)((int)((unsigned)e.mult * (unsigned)acc[t][s][r] + (unsigned)ll[r]) >> e.shift);
-              packed[s][t] = ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
-            } else {
-#pragma unroll
-              for (int r = 0; r < 4; r++) x[r] = (acc[t][s][r] + (int)ll[r]) >> e.shift;
-              packed[s][t] = ashr_sat_pack4(x[0], x[1], x[2], x[3], 0);
-            }
-          }
+          for (int s = 0; s < TM; s++) packed[s][t] = igr_requant4<MODE, FORM>(acc[t][s], kk, ll, e);
         }
       };
 #if PULPNN_BN_BITS == 64
