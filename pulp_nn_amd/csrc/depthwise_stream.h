@@ -46,7 +46,7 @@ __device__ __forceinline__ void dws_wait_vm(int n)
 
 // Preconditions (checked by the host): W % 4 == 0, Wo % 4 == 0, Wo / 4 computing waves (at most 14) plus
 // DWS_LOADERS loader waves per workgroup, CH % 64 == 0, input and output 4-byte aligned, B * CH * H * W < 2^31,
-// PL as the template says; g.NR rows per chunk with g.NR * W % 16 == 0, g.RB chunk slots per channel, g.CSD odd
+// PL as the template says; g.NR rows per chunk with g.NR * W % 16 == 0 and g.NR * W <= 1024, g.RB chunk slots per channel, g.CSD odd
 // and at least g.RB * g.NR * W / 4 dwords, 4 * (64 * g.CSD + 8 * computing waves) bytes of LDS; g.cgroups =
 // CH / 64, g.bands bands of output rows (every band at least one row; one band is the whole plane),
 // g.total = B * g.bands * g.cgroups workgroups.
@@ -89,18 +89,16 @@ __global__ __launch_bounds__(1024, 8) void dw3x3_stream_kernel(DwGeom g, EpiArgs
     const int lw = wave - nwc;
     const __amdgpu_buffer_rsrc_t rsrc_in =
         __builtin_amdgcn_make_buffer_rsrc((void *)g.in, 0, (unsigned)(g.planes * g.H * g.W), 0x00020000);
-    const int chunk_bytes = CR * g.W;
+    // (one instruction per channel and chunk: the host keeps a chunk within the 1 KB a wave's load covers)
     auto request = [&](int k) {
       const int slot = k % NSL;
-      for (int pass = 0; pass * 1024 < chunk_bytes; pass++) {
-        const int off = pass * 1024 + 16 * lane;
-        if (off < chunk_bytes) {
+      const int bytes = min(CR, nreal - k * CR) * g.W;  // the last chunk may be short: nothing is fetched past it
+      if (16 * lane < bytes) {
 #pragma unroll 4
-          for (int c = lw; c < DW_CG; c += DWS_LOADERS) {
-            const int soff = ((b * g.CH + c0 + c) * g.H + iy0 + k * CR) * g.W;
-            unsigned *dst = dw_lds + c * g.CSD + slot * (CR * LWD) + pass * 256;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)dst, 16, off, soff, 0, DWS_AUX);
-          }
+        for (int c = lw; c < DW_CG; c += DWS_LOADERS) {
+          const int soff = ((b * g.CH + c0 + c) * g.H + iy0 + k * CR) * g.W;
+          unsigned *dst = dw_lds + c * g.CSD + slot * (CR * LWD);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)dst, 16, 16 * lane, soff, 0, DWS_AUX);
         }
       }
     };
@@ -109,7 +107,7 @@ __global__ __launch_bounds__(1024, 8) void dw3x3_stream_kernel(DwGeom g, EpiArgs
     // the chunk is consumed, that is behind the next barrier, so chunk k - 1 + NSL is requested behind barrier k.
     // Before this wave arrives at barrier k, chunk k has landed: loads return in order, so that is "at most the
     // requests of the chunks behind k are outstanding", a request being `per` instructions for this wave.
-    const int per = ((chunk_bytes + 1023) / 1024) * ((DW_CG - lw + DWS_LOADERS - 1) / DWS_LOADERS);
+    const int per = (DW_CG - lw + DWS_LOADERS - 1) / DWS_LOADERS;
     int next = min(NSL, nck);
     for (int k = 0; k < next; k++) request(k);
     for (int k = 0; k < nck; k++) {

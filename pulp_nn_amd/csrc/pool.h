@@ -70,8 +70,10 @@ __global__ __launch_bounds__(256) void maxpool_kernel(PoolGeom g)
 }
 
 // Same, 16 channels per thread with 16-byte accesses (C % 16 == 0, 16-byte aligned maps).
-// g.cgroups counts groups of 16 here.
-template <bool NT>
+// g.cgroups counts groups of 16 here.  NT: non-temporal store; LNT: non-temporal loads (windows that do not
+// overlap on an input too large for the caches: every byte is read once).  A whole 2 x 2 window is four loads
+// issued together; other windows go tap by tap.
+template <bool NT, bool LNT>
 __global__ __launch_bounds__(256) void maxpool16_kernel(PoolGeom g)
 {
   long long t = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -85,15 +87,26 @@ __global__ __launch_bounds__(256) void maxpool16_kernel(PoolGeom g)
   const int xs = max(ox * g.sx - g.pl, 0), xe = min(ox * g.sx - g.pl + g.kx, g.W);
   const int ys = max(oy * g.sy - g.pt, 0), ye = min(oy * g.sy - g.pt + g.ky, g.H);
   const uint8_t *img = g.in + (long long)b * g.H * g.W * g.C + cg * 16;
+  auto ld = [&](const uint8_t *p) { return LNT ? __builtin_nontemporal_load((const v4i *)p) : *(const v4i *)p; };
+  auto vmax = [&](v4i &m, const v4i &v) {
+    m.x = (int)max_u8x4((unsigned)m.x, (unsigned)v.x);
+    m.y = (int)max_u8x4((unsigned)m.y, (unsigned)v.y);
+    m.z = (int)max_u8x4((unsigned)m.z, (unsigned)v.z);
+    m.w = (int)max_u8x4((unsigned)m.w, (unsigned)v.w);
+  };
   v4i m = {0, 0, 0, 0};
-  for (int y = ys; y < ye; y++)
-    for (int x = xs; x < xe; x++) {
-      const v4i v = *(const v4i *)(img + ((long long)y * g.W + x) * g.C);
-      m.x = (int)max_u8x4((unsigned)m.x, (unsigned)v.x);
-      m.y = (int)max_u8x4((unsigned)m.y, (unsigned)v.y);
-      m.z = (int)max_u8x4((unsigned)m.z, (unsigned)v.z);
-      m.w = (int)max_u8x4((unsigned)m.w, (unsigned)v.w);
-    }
+  if (ye - ys == 2 && xe - xs == 2) {
+    const uint8_t *p = img + ((long long)ys * g.W + xs) * g.C;
+    const long long row = (long long)g.W * g.C;
+    const v4i v0 = ld(p), v1 = ld(p + g.C), v2 = ld(p + row), v3 = ld(p + row + g.C);
+    m = v0;
+    vmax(m, v1);
+    vmax(m, v2);
+    vmax(m, v3);
+  } else {
+    for (int y = ys; y < ye; y++)
+      for (int x = xs; x < xe; x++) vmax(m, ld(img + ((long long)y * g.W + x) * g.C));
+  }
   store16<NT>(g.out + (((long long)b * g.Ho + oy) * g.Wo + ox) * g.C + cg * 16, m);
 }
 

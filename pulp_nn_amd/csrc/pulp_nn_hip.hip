@@ -582,10 +582,14 @@ void depthwise_common(const char *fn, const uint8_t *in, const int8_t *bias, uin
                      Ho <= (H - 1) / sy + 1 && CH % 4 == 0 && ((long long)g_batch * CH) % DW_CG == 0 && aligned(in, hwc_in ? 4 : 16) &&
                      aligned(out, 4) && (long long)g_batch * CH / DW_CG * Ho < 0x7fffffffLL;
   // Layers that fill the machine with one workgroup per image and 64 channels (two per compute unit): the plane
-  // streamed through LDS, 8 rows of it per request.  Up to 14 groups of 4 output columns, 64 KiB of LDS.
+  // streamed through LDS, 8 rows of it per request.  Up to 14 groups of 4 output columns, 64 KiB of LDS.  A chunk
+  // costs a barrier and a round trip to memory however few rows it holds, so at stride 1 (where the band kernel is
+  // within 3 %) only planes of whole chunks take this kernel: 56 rows do, the 58 pre-padded rows of
+  // pulp_nn_depthwise_3x3_s1 run 7 % faster in bands.
   const int stream_csd = (2 * DWS_ROWS * (W / 4)) | 1;
   const size_t stream_lds = 4 * ((size_t)DW_CG * stream_csd + 8 * (size_t)(Wo / 4));
-  const bool stream = !plane && !rowsk && !hwc_in && lin_dma_ok && Wo / 4 <= 16 - DWS_LOADERS && stream_lds <= 64 * 1024 &&
+  const bool stream = !plane && !rowsk && !hwc_in && lin_dma_ok && Wo / 4 <= 16 - DWS_LOADERS && stream_lds <= 64 * 1024 && DWS_ROWS * W <= 1024 &&
+                      (sx == 2 || H % DWS_ROWS == 0) &&
                       (long long)g_batch * (CH / DW_CG) >= 2ll * num_cus();
   if (hwc_in && !plane && !rowsk)
     return set_error(PULP_NN_HIP_ERR_UNSUPPORTED, fn, "no fused kernel for this geometry: use pulp_nn_hip_hwc_to_chw and the CHW entry point");
@@ -1019,8 +1023,14 @@ void pulp_nn_maxpool(uint8_t *Im_in, uint8_t *Im_out, uint16_t dim_im_in_x, uint
     g.cgroups = ch_im_in / 16;
     g.total = (long long)g.B * g.Ho * g.Wo * g.cgroups;
     const dim3 grid((unsigned)((g.total + 255) / 256));
-    if (g.total * 16 >= PULPNN_NT_BYTES) hipLaunchKernelGGL(maxpool16_kernel<true>, grid, dim3(256), 0, g_stream, g);
-    else hipLaunchKernelGGL(maxpool16_kernel<false>, grid, dim3(256), 0, g_stream, g);
+    // non-temporal loads: windows that do not overlap, on an input too large to find again in a cache
+    const bool lnt = stride_x >= dim_kernel_x && stride_y >= dim_kernel_y &&
+                     (long long)g.B * g.H * g.W * g.C >= PULPNN_NT_BYTES;
+    const bool snt = g.total * 16 >= PULPNN_NT_BYTES;
+    if (snt && lnt) hipLaunchKernelGGL((maxpool16_kernel<true, true>), grid, dim3(256), 0, g_stream, g);
+    else if (snt) hipLaunchKernelGGL((maxpool16_kernel<true, false>), grid, dim3(256), 0, g_stream, g);
+    else if (lnt) hipLaunchKernelGGL((maxpool16_kernel<false, true>), grid, dim3(256), 0, g_stream, g);
+    else hipLaunchKernelGGL((maxpool16_kernel<false, false>), grid, dim3(256), 0, g_stream, g);
   } else {
     hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((g.total + 255) / 256)), dim3(256), 0, g_stream, g);
   }

@@ -161,14 +161,16 @@ DW_GEOMS = [
     (1, 64, 11, 16, 3, 3, (1, 1, 1, 1), (1, 1)),     # ... height not a multiple of the rows per lane
     (2, 32, 9, 32, 3, 3, (1, 1, 1, 1), (2, 2)),      # ... stride 2, odd height
     (1, 64, 12, 16, 3, 3, (1, 0, 1, 1), (1, 1)),     # ... no bottom padding: one output row fewer
-    # 512 or more (image, 64 channels) units: whole planes streamed through LDS in chunks of 8 rows
-    (64, 512, 12, 12, 3, 3, (1, 1, 1, 1), (1, 1)),   # two chunks, the second partly filled
-    (16, 2048, 19, 8, 3, 3, (1, 1, 1, 1), (1, 1)),   # three chunks, two groups of columns (both at an edge)
-    (16, 2048, 9, 24, 3, 3, (1, 1, 1, 1), (2, 2)),   # stride 2, odd height
-    (64, 512, 11, 12, 3, 3, (0, 1, 0, 2), (1, 1)),   # no top / left padding, two columns of right padding
+    # 512 or more (image, 64 channels) units: whole planes streamed through LDS in chunks of 8 rows (at stride 1
+    # only planes of whole chunks)
+    (64, 512, 16, 12, 3, 3, (1, 1, 1, 1), (1, 1)),   # two chunks
+    (16, 2048, 24, 8, 3, 3, (1, 1, 1, 1), (1, 1)),   # three chunks, two groups of columns (both at an edge)
+    (16, 2048, 9, 24, 3, 3, (1, 1, 1, 1), (2, 2)),   # stride 2, odd height: the second chunk is one row
+    (64, 512, 8, 12, 3, 3, (0, 1, 0, 2), (1, 1)),    # no top / left padding, two columns of right padding
     (32, 1024, 13, 24, 3, 3, (0, 0, 0, 1), (2, 2)),  # stride 2 without top / left padding
-    (64, 512, 10, 12, 3, 3, (2, 0, 1, 1), (1, 1)),   # two rows of top padding, none at the bottom
-    (8, 4096, 17, 16, 3, 3, (1, 1, 0, 2), (1, 1)),   # 16-byte rows that the register kernel does not take (pl = 0)
+    (64, 512, 16, 12, 3, 3, (2, 0, 1, 1), (1, 1)),   # two rows of top padding, none at the bottom
+    (8, 4096, 16, 16, 3, 3, (1, 1, 0, 2), (1, 1)),   # 16-byte rows that the register kernel does not take (pl = 0)
+    (64, 512, 12, 12, 3, 3, (1, 1, 1, 1), (1, 1)),   # stride 1, 12 rows: not whole chunks, the band kernel
 ]
 
 
