@@ -284,7 +284,7 @@ def main():
                                                 56, 56, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1, 2, 2, 1, 1)
                 want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
                                                 (1, 1, 1, 1), (2, 2), 1, 1, 32)
-                kern = "dw3x3_lin_kernel<2, 1, 0, true, true>"
+                kern = "dw3x3_stream_kernel<2, 1, 0>"
             wall, dev, tm = time_launches(step_c2, steps, warm)
             layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev, tm,
                          np.array_equal(outs2[0][:2].cpu().numpy(), want), "hbm", kern)
@@ -310,7 +310,7 @@ def main():
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
         layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev, tm,
                      np.array_equal(outs4[0][:1].cpu().numpy(), want), "mfma",
-                     "igemm_ring_kernel<0, 4, 0> (persistent workgroups on 256 x 256 tiles, LDS-direct loads)",
+                     "igemm_patch_kernel<0, 0> (persistent workgroups on patches of 4 x 64 pixels x 256 channels, LDS-direct loads)",
                      note="random int8 operands: the matrix cores alone sustain 3.6-4.0 POP/s on this data (the clock "
                           "drops under the power limit: profiles/mfma_ceiling.txt); where this kernel's time goes, part "
                           "by part: profiles/conv_cfg4_phases_ablation.txt")
@@ -325,7 +325,7 @@ def main():
         want = oracle.maxpool(outs4[0][:2].cpu().numpy(), (2, 2), (2, 2), out_hw=(32, 32))
         mp_bytes = 64 * (63 * 63 * 256 + 32 * 32 * 256)
         layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev, tm,
-                     np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", "maxpool16_kernel<false>")
+                     np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", "maxpool16_kernel<false, true>")
         gen = torch.Generator(device="cuda")
         gen.manual_seed(20244)
         vec = torch.randint(0, 256, (64, 1024), dtype=torch.uint8, device="cuda", generator=gen)

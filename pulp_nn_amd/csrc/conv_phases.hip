@@ -209,7 +209,7 @@ int main()
     fflush(stdout);
     if (bad) return 1;
   }
-  printf("-- 4 x 64 pixel patches, input rows staged once per filter row (igemm_patch_kernel; the library's kernel for this layer) --\n");
+  printf("-- 4 x 64 pixel patches, input rows staged once per filter row (igemm_patch_kernel: the library's kernel for this layer) --\n");
   run<0, 0>("complete", g, e, dtr, true);
   run<0, 1>("no loads behind a tile's first two groups", g, e, dtr, false);
   run<0, 4>("no fragment reads in the loop", g, e, dtr, false);
@@ -217,7 +217,7 @@ int main()
   run<0, 32>("activation loads out of range (zeros, no traffic)", g, e, dtr, false);
   run<0, 64>("weight loads out of range", g, e, dtr, false);
   run<0, 96>("all loads out of range", g, e, dtr, false);
-  printf("-- 256 consecutive pixels x 256 channels, one sub-slice per tap (igemm_ring_kernel) --\n");
+  printf("-- 256 consecutive pixels x 256 channels, one sub-slice per tap (igemm_ring_kernel: the library's kernel for other shapes) --\n");
   run<4, 0>("complete", g, e, dtr, true);
   run<4, 1>("no loads behind a tile's first sub-slices", g, e, dtr, false);
   run<4, 4>("no fragment reads in the loop", g, e, dtr, false);

@@ -26,16 +26,16 @@
 //     current sub-slice is read into the registers of fragment s when that one's MFMAs are issued, fragment s of
 //     the next sub-slice into those of fragment s + 4: every read is four MFMA groups (64 MFMAs of the two waves
 //     of a SIMD) ahead of its use.
-// Output pixels outside the image (column 63 when Wo = 63, rows past Ho) are computed and not stored.
+// Output pixels outside the image (column 63 when Wo = 63, rows past Ho) are computed and not stored; the host
+// takes this kernel only when at least nine tenths of the patch grid are real pixels.
 //
-// A measurement variant: the library does not launch this kernel, the conv_phases tool does, next to
-// igemm_ring_kernel and with byte-for-byte equal output.  On the 64 x 64 x 256 -> 256 layer at batch 64 it fetches
-// 31 % fewer bytes from L2 and spends 3 % less time in the main loop, and the launch as a whole is within 1 % of
-// igemm_ring_kernel's (139 against 139 to 140 us on the same machine): the layer runs at the power limit (shader
-// clock 2.0 to 2.1 GHz inside the loop against 2.4 GHz for the same loop on zeros), and what the saved traffic
-// gives back is of the size of the difference between two machines.  Preconditions: kx = 3, stride 1, pl <= 1,
-// Wo <= 64, ky <= 31, ky * Ci / 64 >= 2 groups, Ci % 64 = 0, N % 16 = 0, whole images, a grid that is a multiple
-// of 8 * tiles_n and no larger than the number of tiles, g.rgroups = ceil(Ho / 4) with its divisor.
+// Measured on the 64 x 64 x 256 -> 256 layer at batch 64 (conv_phases tool, both kernels in one run, output equal byte
+// for byte): 31 % fewer bytes from L2, 3 % less time in the main loop, the launch 1 to 2 % shorter than
+// igemm_ring_kernel's (142 against 144 us).  The layer runs at the power limit (shader clock 2.0 to 2.1 GHz inside
+// the loop against 2.4 GHz for the same loop on zeros), so the saved traffic comes back as a little more clock.
+// Preconditions (checked by the host): kx = 3, stride 1, pl <= 1, Wo <= 64, ky <= 31, ky * Ci / 64 >= 2 groups,
+// Ci % 64 = 0, N % 16 = 0, whole images, a grid that is a multiple of 8 * tiles_n and no larger than the number of
+// tiles, g.rgroups = ceil(Ho / 4) with its divisor.
 #pragma once
 #include "igemm_ring.h"
 
@@ -58,12 +58,11 @@ static inline int igp_lds_bytes() { return IGP_DUMP_AT + IGP_DUMP + IGP_BN * (4 
 template <int MODE, int ABL = 0>
 __global__ __launch_bounds__(IGP_THREADS, 1) void igemm_patch_kernel(ConvGeom g, EpiArgs e)
 {
-  constexpr int TM = 8, TN = 4, WM = 128, WNC = 64, BN = IGP_BN, GA = 3, GW = 2;
+  constexpr int TM = 8, TN = 4, WNC = 64, BN = IGP_BN, GA = 3, GW = 2;
   constexpr int G = GA + 3 * GW;  // loads per wave and group
   typedef __attribute__((address_space(3))) void *lds_ptr_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char igr_lds[];
-  unsigned char *dump = igr_lds + IGP_DUMP_AT;
-  int *wsum = (int *)(dump + IGP_DUMP);  // weight sums by LDS row
+  int *wsum = (int *)(igr_lds + IGP_DUMP_AT + IGP_DUMP);  // weight sums by LDS row
   bn_t *cadd = (bn_t *)(wsum + BN);      // per channel: additive constant of the epilogue
   bn_t *cmul = cadd + BN;                // per channel: multiplier (batch-norm branch)
 
@@ -141,11 +140,10 @@ __global__ __launch_bounds__(IGP_THREADS, 1) void igemm_patch_kernel(ConvGeom g,
     const int fy_s = __builtin_amdgcn_readfirstlane((int)fy);
     const int soff_a = __builtin_amdgcn_readfirstlane((int)(fy * (unsigned)g.W * (unsigned)g.Ci + ci));
     const int soff_w = __builtin_amdgcn_readfirstlane((int)(fy * (unsigned)g.kx * (unsigned)g.Ci + ci));
-    unsigned char *base = igr_lds + u_a * IGP_A_BYTES;
 #pragma unroll
     for (int j = 0; j < GA; j++) {
       const int beta = wave + 8 * j;
-      unsigned char *dst = beta < IGP_A_BLOCKS ? base + 1024 * beta : dump;
+      unsigned char *dst = igr_lds + (beta < IGP_A_BLOCKS ? u_a * IGP_A_BYTES + 1024 * beta : IGP_DUMP_AT);
       const unsigned oob = ((unsigned)__builtin_amdgcn_sbfe((int)pinv[j], fy_s, 1) & OOB) | dead | ((ABL & 32) ? OOB : 0u);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)dst, 16, (int)(poff[j] | oob), soff_a, 0, 0);
     }
@@ -332,9 +330,8 @@ __global__ __launch_bounds__(IGP_THREADS, 1) void igemm_patch_kernel(ConvGeom g,
       // (the table offset of this lane is made opaque: the 32 table addresses it leads to are then one register plus
       // immediates, computed here; known to be loop-invariant they are computed before the tile loop, each in a
       // register of its own, and spilled)
-      unsigned cb_bytes = (unsigned)cb * (unsigned)sizeof(bn_t);
-      asm volatile("" : "+v"(cb_bytes));
-      const bn_t *ctab = (const bn_t *)((const unsigned char *)cadd + cb_bytes);
+      int cbo = cb;
+      asm volatile("" : "+v"(cbo));
       unsigned packed[TM][TN];
       auto requantise = [&](auto form_tag) {
         constexpr int FORM = decltype(form_tag)::value;
@@ -343,8 +340,8 @@ __global__ __launch_bounds__(IGP_THREADS, 1) void igemm_patch_kernel(ConvGeom g,
           bn_t kk[4], ll[4];
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            ll[r] = ctab[4 * t + r];
-            kk[r] = MODE == EPI_BN ? ctab[BN + 4 * t + r] : (bn_t)0;
+            ll[r] = cadd[cbo + 4 * t + r];
+            kk[r] = MODE == EPI_BN ? cmul[cbo + 4 * t + r] : (bn_t)0;
           }
 #pragma unroll
           for (int s = 0; s < TM; s++) packed[s][t] = igr_requant4<MODE, FORM>(acc[t][s], kk, ll, e);
@@ -354,7 +351,7 @@ __global__ __launch_bounds__(IGP_THREADS, 1) void igemm_patch_kernel(ConvGeom g,
       if constexpr (MODE == EPI_BN) {
         bool ks = true;
 #pragma unroll
-        for (int c = 0; c < 16; c++) ks = ks && bn_k_small(ctab[BN + c]);
+        for (int c = 0; c < 16; c++) ks = ks && bn_k_small(cmul[cbo + c]);
         const bool small = __all(ks);  // wave-uniform
         if (small && e.shift >= 32) requantise(std::integral_constant<int, 0>{});
         else if (small) requantise(std::integral_constant<int, 1>{});

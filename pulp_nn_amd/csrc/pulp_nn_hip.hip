@@ -25,6 +25,7 @@
 #include "dwpw_fused.h"
 #include "igemm.h"
 #include "igemm_ring.h"
+#include "igemm_patch.h"
 #include "depthwise_stream.h"
 #include "linear_skinny.h"
 #include "pool.h"
@@ -188,6 +189,50 @@ bool launch_igemm_ring(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   return true;
 }
 
+// 4-row x 64-column output patches whose input rows are staged once per filter row (igemm_patch.h): 3-wide
+// stride-1 filters on images of 57 to 64 output columns.  Returns false if the shape does not qualify.
+bool launch_igemm_patch(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
+{
+  if (g.kx != 3 || g.sx != 1 || g.sy != 1 || g.pl > 1 || g.Wo > 64 || g.ky > 31) return false;
+  if (g.Ci % 64 || g.ky * (g.Ci / 64) < 2 || g.K >= 65536 || g.N % 16 || !aligned(g.out, 16) || mode == EPI_OUT32) return false;
+  if (g.M % g.HoWo) return false;  // whole images
+  // pixels wanted against pixels computed (whole patches): at least nine tenths
+  const int rgroups = (g.Ho + 3) / 4;
+  if ((long long)g.Ho * g.Wo * 10 < (long long)rgroups * 4 * 64 * 9) return false;
+  g.tiles_n = (g.N + IGP_BN - 1) / IGP_BN;
+  conv_geom_divs(g);
+  g.rgroups = rgroups;
+  g.d_rg = fastdiv_make((unsigned)rgroups);
+  const long long tiles = (long long)g.batch * rgroups * g.tiles_n;
+  if (tiles > 0x7fffffffLL) return false;
+  g.tiles_total = (int)tiles;
+  const int unit = 8 * g.tiles_n;
+  const int grid_n = (int)(std::min<long long>(num_cus(), g.tiles_total) / unit) * unit;
+  if (grid_n <= 0) return false;
+  g.cpt = g.Ci / 64;
+  g.d_cpt = fastdiv_make((unsigned)g.cpt);
+  g.d_kx = fastdiv_make((unsigned)g.kx);
+  g.vec_store = 1;
+  g.nt = (long long)g.M * g.N >= PULPNN_NT_BYTES;
+  const size_t lds = (size_t)igp_lds_bytes();
+  const dim3 grid(grid_n), block(IGP_THREADS);
+  switch (mode) {
+    case EPI_BN:
+      if (!raise_lds_limit<igemm_patch_kernel<EPI_BN>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_patch_kernel<EPI_BN>), grid, block, lds, s, g, e);
+      break;
+    case EPI_MULT:
+      if (!raise_lds_limit<igemm_patch_kernel<EPI_MULT>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_patch_kernel<EPI_MULT>), grid, block, lds, s, g, e);
+      break;
+    default:
+      if (!raise_lds_limit<igemm_patch_kernel<EPI_RAW>>(lds)) return false;
+      hipLaunchKernelGGL((igemm_patch_kernel<EPI_RAW>), grid, block, lds, s, g, e);
+      break;
+  }
+  return true;
+}
+
 // 128 px x 64 ch tiles, for layers too small to fill the machine with larger ones.  With at most five
 // K slices (K <= 320) a tile's whole K extent fits in LDS and is fetched in one go.
 template <int GATHER>
@@ -205,6 +250,7 @@ void launch_igemm_tile(int mode, ConvGeom &g, const EpiArgs &e, hipStream_t s)
   const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N + 255) / 256);
   if (GATHER == GATHER_UNIFORM && g.N > 128 && big_tiles >= 2 * num_cus()) {
     // operands go HBM/L2 -> LDS without passing through registers, persistent workgroups
+    if (launch_igemm_patch(mode, g, e, s)) return;
     if (launch_igemm_ring(mode, g, e, s)) return;
     launch_igemm_mode<4, 4, 4, GATHER>(mode, g, e, s);
   } else

@@ -4,7 +4,8 @@ That path is taken by convolutions with input channels a multiple of 64, more th
 of 16), K of at least 256 bytes and at least two 256 x 256 tiles per compute unit; these geometries are sized to reach
 it and to exercise its edges (channel tail, pixel tail, padding on every side, stride 2, several channel tiles, an
 odd number of K sub-slices, the shortest K, every epilogue branch, both widths).  One geometry (136 channels) stays
-on the tiled kernel of the same tile size."""
+on the tiled kernel of the same tile size.  3-wide stride-1 filters on images of 57 to 64 output columns take the
+patch-tiled variant of the path (4 x 64 pixel patches, input rows staged once per filter row); five geometries reach it."""
 import numpy as np
 import pytest
 
@@ -22,6 +23,13 @@ GEOMS = [
     (84, 40, 40, 64, 256, 3, 3, (1, 1, 1, 1), (1, 1)),      # 64 input channels: one K sub-slice per tap, nine in all (odd)
     (70, 48, 48, 192, 512, 3, 3, (1, 1, 1, 1), (1, 1)),     # two channel tiles per pixel tile, three sub-slices per tap
     (262, 23, 23, 320, 256, 1, 1, (0, 0, 0, 0), (1, 1)),    # K = 320: five sub-slices, one more than the ring has stages
+    # 3-wide stride-1 filters on 57 to 64 output columns: patches of 4 rows x 64 columns, input rows staged once per
+    # filter row (igemm_patch_kernel)
+    (36, 62, 60, 64, 256, 3, 3, (1, 1, 1, 1), (1, 1)),      # 60 columns, 62 rows (two dead rows in the last patch), one group per filter row
+    (34, 64, 64, 128, 512, 3, 3, (1, 0, 1, 0), (1, 1)),     # config 4 shape (63 x 63 out), two channel tiles
+    (40, 60, 64, 128, 192, 1, 3, (0, 0, 1, 1), (1, 1)),     # 1 x 3 filter: two groups in all; channel tail
+    (34, 64, 64, 64, 256, 5, 3, (2, 2, 0, 1), (1, 1)),      # 5 x 3 filter, no left padding, 63 columns
+    (38, 58, 62, 192, 256, 3, 3, (0, 1, 1, 0), (1, 1)),     # no top padding, three groups per filter row, 57 x 61 out
 ]
 FLAGS = [(1, 1), (1, 0), (0, 0), (0, 1)]
 
