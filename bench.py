@@ -40,6 +40,32 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA, op/s
 PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_all_layers_hbm_traffic.txt")
+TRACE_FILE = os.path.join(ROOT, "profiles", "bench_all_layers_kernel_trace.txt")
+# The kernel each workload is expected to dispatch to.  The library does not report what it launched, so these
+# names are checked against the committed kernel trace of this same benchmark (tests/test_bench_kernels.py, and
+# `kernel_in_committed_trace` in every roofline object): a dispatch rule that changes without the profiles being
+# regenerated shows up there.
+KERNELS = {
+    "cfg1_pointwise": "pw_stream_kernel<4, 2, 4, 1, true, 1, 16>",
+    "cfg0_conv": "igemm_kernel<2, 2, 2, 3, 0, 4, 5>",
+    "cfg2_dw_s1": "dw3x3_lin_kernel<1, 1, 0, true, true>",
+    "cfg2_dw_s2": "dw3x3_stream_kernel<2, 1, 0>",
+    "cfg4_conv": "igemm_patch_kernel<0, 0>",
+    "cfg4_maxpool": "maxpool16_kernel<false, true>",
+    "cfg4_linear": "linear_skinny_kernel<0>",
+}
+
+
+def traced_kernels():
+    """Kernel names (up to the argument list) of the committed kernel-trace summary; empty if it is missing."""
+    if not os.path.exists(TRACE_FILE):
+        return set()
+    names = set()
+    for line in open(TRACE_FILE):
+        m = re.match(r"^(?:void )?(\w+(?:<.*?>)?)\(", line)
+        if m:
+            names.add(m.group(1))
+    return names
 
 
 def profiled_traffic():
@@ -85,6 +111,7 @@ def main():
     for L in libs.values():
         L.use_torch_stream()     # the library queues on torch's current stream, which the events below time
     traffic = profiled_traffic()
+    traced = traced_kernels()
     failures = []
 
     def t(a):
@@ -145,6 +172,7 @@ def main():
         # that kernel has no line there)
         r["traffic"] = traffic_for(traffic, kernel.split("(")[0].strip())
         r["traffic_measured_in_this_run"] = False
+        r["kernel_in_committed_trace"] = kernel.split("(")[0].strip() in traced
         return r
 
     # ---- headline: config 1 -------------------------------------------------
@@ -176,7 +204,7 @@ def main():
         failures.append("configs[1] pointwise")
 
     gops = c1["ops"] / (wall_ms * 1e-3) / 1e9
-    head_kernel = "pw_stream_kernel<4, 2, 4, 1, true, 1, 16>"
+    head_kernel = KERNELS["cfg1_pointwise"]
     rec = {
         "metric": "int8 GOPS and % int8 MFMA peak per conv layer at batch 256; bit-exact",
         "value": round(gops, 1),
@@ -213,6 +241,7 @@ def main():
             "traffic": traffic_for(traffic, head_kernel),
             "traffic_source": "profiles/bench_all_layers_hbm_traffic.txt",
             "traffic_measured_in_this_run": False,
+            "kernel_in_committed_trace": head_kernel in traced,
         },
     }
 
@@ -255,7 +284,7 @@ def main():
                            c0["strides"], 1, 1, 32)
         layer_record(c0["name"] + "_b256", c0["ops"], c0["bytes"], wall, dev, tm,
                      np.array_equal(outs0[0][:8].cpu().numpy(), want), "mfma",
-                     "igemm_kernel<2, 2, 2, 3, 0, 4, 5> (128 x 64 tiles, whole K in one pass)",
+                     KERNELS["cfg0_conv"] + " (128 x 64 tiles, whole K in one pass)",
                      note="6.3 MB and 2.4 GOP per launch: bound by launch and memory latency, not by a pipe")
         del xs0, outs0
 
@@ -276,7 +305,7 @@ def main():
                     L.pulp_nn_depthwise_3x3_s1(xs2[j], outs2[j], 58, 56, 128, 1, 1, w2, c2["out_shift"], 0, k2, l2,
                                                1, 1, None)
                 want = oracle.depthwise_3x3_s1(xin[:2], c2["w"], c2["k"], c2["lam"], 0, c2["out_shift"], 1, 1, 1, 1, 32)
-                kern = "dw3x3_lin_kernel<1, 1, 0, true, true>"
+                kern = KERNELS["cfg2_dw_s1"]
             else:
                 def step_c2(i):
                     j = i % nset
@@ -284,7 +313,7 @@ def main():
                                                 56, 56, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1, 2, 2, 1, 1)
                 want = oracle.depthwise_generic(xin[:2], c2["w"], c2["bias"], c2["k"], c2["lam"], 0, c2["out_shift"],
                                                 (1, 1, 1, 1), (2, 2), 1, 1, 32)
-                kern = "dw3x3_stream_kernel<2, 1, 0>"
+                kern = KERNELS["cfg2_dw_s2"]
             wall, dev, tm = time_launches(step_c2, steps, warm)
             layer_record(c2["name"] + "_b256", c2["ops"], c2["bytes"], wall, dev, tm,
                          np.array_equal(outs2[0][:2].cpu().numpy(), want), "hbm", kern)
@@ -310,7 +339,7 @@ def main():
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
         layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev, tm,
                      np.array_equal(outs4[0][:1].cpu().numpy(), want), "mfma",
-                     "igemm_patch_kernel<0, 0> (persistent workgroups on patches of 4 x 64 pixels x 256 channels, LDS-direct loads)",
+                     KERNELS["cfg4_conv"] + " (persistent workgroups on patches of 4 x 64 pixels x 256 channels, LDS-direct loads)",
                      note="random int8 operands: the matrix cores alone sustain 3.6-4.0 POP/s on this data (the clock "
                           "drops under the power limit: profiles/mfma_ceiling.txt); where this kernel's time goes, part "
                           "by part: profiles/conv_cfg4_phases_ablation.txt")
@@ -325,7 +354,7 @@ def main():
         want = oracle.maxpool(outs4[0][:2].cpu().numpy(), (2, 2), (2, 2), out_hw=(32, 32))
         mp_bytes = 64 * (63 * 63 * 256 + 32 * 32 * 256)
         layer_record("cfg4_maxpool2x2_s2_63x63x256_b64", 0, mp_bytes, wall, dev, tm,
-                     np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", "maxpool16_kernel<false, true>")
+                     np.array_equal(pooled[0][:2].cpu().numpy(), want), "hbm", KERNELS["cfg4_maxpool"])
         gen = torch.Generator(device="cuda")
         gen.manual_seed(20244)
         vec = torch.randint(0, 256, (64, 1024), dtype=torch.uint8, device="cuda", generator=gen)
@@ -339,7 +368,7 @@ def main():
         want = oracle.linear(vec.cpu().numpy(), c4["lin_w"], c4["lin_bias"], c4["lin_k"], c4["lin_lam"], 0,
                              c4["lin_shift"], 1, 1, 64)
         layer_record("cfg4_linear_1024_4096_b64", 2 * 64 * 1024 * 4096, 64 * (1024 + 4096) + 4096 * 1024 + 4096 * 17,
-                     wall, dev, tm, np.array_equal(lout.cpu().numpy(), want), "hbm", "linear_skinny_kernel<0>",
+                     wall, dev, tm, np.array_equal(lout.cpu().numpy(), want), "hbm", KERNELS["cfg4_linear"],
                      note="4.5 MB per launch: bound by launch and memory latency")
         del xs4, outs4, pooled
 
