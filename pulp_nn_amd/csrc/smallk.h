@@ -147,6 +147,7 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
   __shared__ __attribute__((aligned(16))) int wl[NCH * SMALLK_RP];  // [channel][row][dword]
   __shared__ int corr_l[NCH];
   __shared__ bn_t k_l[NCH], lam_l[NCH];
+  __shared__ int k_small_l;
 
   const int tid = threadIdx.x;
   const int L = g.kx * g.Ci;  // bytes per filter row
@@ -170,12 +171,18 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
     for (int d = 0; d < 3 * SMALLK_RD; d++) sum = __builtin_amdgcn_sdot4(wl[tid * SMALLK_RP + d], 0x01010101, sum, false);
     const bool real = tid < g.N;
     corr_l[tid] = 128 * sum + ((real && g.bias) ? (int)g.bias[tid] : 0);
+    bn_t kv = 0;
     if (MODE == EPI_BN) {
-      k_l[tid] = real ? e.k[tid] : 0;
+      kv = real ? e.k[tid] : 0;
+      k_l[tid] = kv;
       lam_l[tid] = real ? e.lambda[tid] : 0;
     }
+    // do all multipliers fit the fast form of the requantisation?  (NCH <= 64: these lanes are one wave)
+    const bool all_small = __all(bn_k_small(kv));
+    if (tid == 0) k_small_l = all_small;
   }
   __syncthreads();
+  const bool k_small = k_small_l != 0;
 
   // ---- this lane's pixels: the (up to) three filter rows of each ---------------------------------
   // A workgroup takes g.tiles_n runs of 256 consecutive pixels (the weight table and the two barriers above are
@@ -250,6 +257,11 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
     finish(cur, a);
 
     // ---- NCH dot products, requantise, store ----------------------------------------------
+    // (the weight table is read through an offset the compiler cannot see through: known to be the same in every
+    // pass, all NCH x 9 weight dwords would be read before the loop and kept in registers, 2 waves per SIMD fit then)
+    int wofs = 0;
+    asm volatile("" : "+s"(wofs));
+    const int *wt = wl + wofs;
     unsigned packed[NCH / 4];
 #pragma unroll
     for (int n4 = 0; n4 < NCH / 4; n4++) {
@@ -258,8 +270,8 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
       for (int r = 0; r < 4; r++) {
         const int n = 4 * n4 + r;
         acc[r] = corr_l[n];
-        const v4i w0 = *(const v4i *)&wl[n * SMALLK_RP], w1 = *(const v4i *)&wl[n * SMALLK_RP + 4];
-        const int w2 = wl[n * SMALLK_RP + 8];
+        const v4i w0 = *(const v4i *)&wt[n * SMALLK_RP], w1 = *(const v4i *)&wt[n * SMALLK_RP + 4];
+        const int w2 = wt[n * SMALLK_RP + 8];
         acc[r] = __builtin_amdgcn_sdot4((int)a[0][0], w0.x, acc[r], false);
         acc[r] = __builtin_amdgcn_sdot4((int)a[0][1], w0.y, acc[r], false);
         acc[r] = __builtin_amdgcn_sdot4((int)a[0][2], w0.z, acc[r], false);
@@ -270,14 +282,15 @@ __global__ __launch_bounds__(256) void smallk_rows_kernel(ConvGeom g, EpiArgs e)
         acc[r] = __builtin_amdgcn_sdot4((int)a[2][1], w1.w, acc[r], false);
         acc[r] = __builtin_amdgcn_sdot4((int)a[2][2], w2, acc[r], false);
       }
-      unsigned p = 0;
+      // four outputs at a time: |acc| < 2^21 here (at most 36 products of a byte and a signed byte, plus the
+      // correction term), so the 24-bit multiplier gives the exact low 32 bits where the multipliers fit 24 bits
+      bn_t kk[4], ll[4];
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const int n = 4 * n4 + r;
-        const bn_t kk = (MODE == EPI_BN) ? k_l[n] : (bn_t)0, ll = (MODE == EPI_BN) ? lam_l[n] : (bn_t)0;
-        p |= (unsigned)requant<MODE>(acc[r], kk, ll, e.mult, e.shift) << (8 * r);
+        kk[r] = (MODE == EPI_BN) ? k_l[4 * n4 + r] : (bn_t)0;
+        ll[r] = (MODE == EPI_BN) ? lam_l[4 * n4 + r] : (bn_t)0;
       }
-      packed[n4] = p;
+      packed[n4] = requant4<MODE, true>(acc[0], acc[1], acc[2], acc[3], kk, ll, k_small, e.mult, e.shift);
     }
     if (m < g.M) {
       uint8_t *o = (uint8_t *)g.out + (long long)m * g.N;
