@@ -46,8 +46,8 @@ __device__ __forceinline__ void dws_wait_vm(int n)
 
 // Preconditions (checked by the host): W % 4 == 0, Wo % 4 == 0, Wo / 4 computing waves (at most 14) plus
 // DWS_LOADERS loader waves per workgroup, CH % 64 == 0, input and output 4-byte aligned, B * CH * H * W < 2^31,
-// PL as the template says; g.NR rows per chunk with g.NR * W % 16 == 0 and g.NR * W <= 1024, g.RB chunk slots per channel, g.CSD odd
-// and at least g.RB * g.NR * W / 4 dwords, 4 * (64 * g.CSD + 8 * computing waves) bytes of LDS; g.cgroups =
+// PL as the template says; g.NR rows per chunk with g.NR * W % 16 == 0 and g.NR * W <= 1024, g.RB chunk slots per
+// channel, g.CSD odd and at least g.RB * g.NR * W / 4 dwords, 4 * (64 * g.CSD + 8 * computing waves) bytes of LDS; g.cgroups =
 // CH / 64, g.bands bands of output rows (every band at least one row; one band is the whole plane),
 // g.total = B * g.bands * g.cgroups workgroups.
 // The stores keep the default cache policy: a workgroup writes 64 of a pixel's channels, half a 128-byte line, and
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(1024, 8) void dw3x3_stream_kernel(DwGeom g, EpiArgs
   const int ipb = o0 * S;
   const int PR = (nho - 1) * S + 3;
   const int iy0 = max(0, ipb - g.pt), ztop = max(0, g.pt - ipb);
-  const int nreal = min(g.H, ipb + PR - g.pt) - iy0;
+  const int nreal = max(0, min(g.H, ipb + PR - g.pt) - iy0);  // (0: a band that lies in the padding altogether)
   const int nck = (nreal + CR - 1) / CR;  // chunks of the band
 
   if (wave >= nwc) {
