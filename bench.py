@@ -117,10 +117,13 @@ def main():
     def t(a):
         return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
-    def time_launches(fn, steps, warmup, min_ms=None, min_repeats=10, max_repeats=4000):
+    probe_buf = torch.zeros((4096, 2), dtype=torch.int64, device="cuda")
+
+    def time_launches(fn, steps, warmup, min_ms=None, min_repeats=10, max_repeats=4000, series=False):
         """fn(i) queues one step on torch's current stream (the library's stream).  Times regions of exactly
         `steps` steps, each between two synchronisations, one after the other; returns (median wall ms per step,
-        median device ms per step from HIP events, timing summary)."""
+        median device ms per step from HIP events, timing summary).  Behind every region the library's clock probe
+        is queued (20 us, outside the timed interval): the shader clock the region left the GPU at."""
         min_ms = (6.0 if args.quick else 60.0) if min_ms is None else min_ms
         for i in range(warmup):
             fn(i)
@@ -135,6 +138,7 @@ def main():
                 fn(it)
                 it += 1
             e1.record()
+            libs[32].clock_probe(probe_buf[len(walls)])
             torch.cuda.synchronize()
             t1 = time.perf_counter()
             walls.append((t1 - t0) * 1e3 / steps)
@@ -152,6 +156,13 @@ def main():
                                           "median_after_first_10ms": round(statistics.median(
                                               devs[min(len(devs) - 1, next((n for n in range(len(devs)) if sum(devs[:n + 1]) * steps >= 10.0),
                                                                             len(devs) - 1)):]) * 1e3, 2)}}
+        pr = probe_buf[:len(devs)].cpu().numpy()
+        mhz = [round(100.0 * float(c) / float(t)) if t else 0 for t, c in pr]
+        summary["shader_mhz_behind_region"] = {"first_region": mhz[0], "min": min(mhz), "median": int(statistics.median(mhz)),
+                                               "max": max(mhz)}
+        if series:
+            # the first regions one by one: [device us per step, shader MHz behind the region]
+            summary["first_regions"] = [[round(d * 1e3, 2), m] for d, m in list(zip(devs, mhz))[:24]]
         return statistics.median(walls), statistics.median(devs), summary
 
     def rotating(nbytes):
@@ -192,7 +203,7 @@ def main():
         L.pulp_nn_pointwise_HoWo_parallel(xs[j], None, bias, outs[j], w, None, None, c1["out_mult"], c1["out_shift"],
                                           W, H, Ci, W, H, Co, 1, 1, 0, 0, 0, 0, 1, 1, c1["relu"], c1["bn"])
 
-    wall_ms, dev_ms, timing = time_launches(step_c1, args.steps, args.warmup)
+    wall_ms, dev_ms, timing = time_launches(step_c1, args.steps, args.warmup, series=True)
 
     # parity of what was just computed, on a sample of the batch (the oracle is the checker, outside the timed region)
     import oracle
@@ -256,6 +267,9 @@ def main():
                 "hbm_frac": round(nbytes / (dev * 1e-3) / PEAK_HBM, 4),
                 "roofline": roofline(bound, ops, nbytes, dev, kernel),
                 "parity": "bit-exact" if ok else "MISMATCH"}
+        rec_["shader_mhz_behind_region"] = tm["shader_mhz_behind_region"]
+        if "first_regions" in tm:
+            rec_["first_regions"] = tm["first_regions"]
         rec_.update(extra)
         layers.append(rec_)
         if not ok:
@@ -334,7 +348,7 @@ def main():
             L4.pulp_nn_conv_Ho_parallel(xs4[j], None, b4, outs4[j], w4, k4, l4, 0, c4["out_shift"], 64, 64, 256, 63, 63,
                                         256, 3, 3, 1, 0, 1, 0, 1, 1, 1, 1)
 
-        wall, dev, tm = time_launches(step_c4, max(5, steps // 4), 2)
+        wall, dev, tm = time_launches(step_c4, max(5, steps // 4), 2, series=True)
         want = oracle.conv(c4["x"][:1], c4["w"], c4["bias"], c4["k"], c4["lam"], 0, c4["out_shift"], c4["pads"],
                            c4["strides"], 1, 1, 64, out_hw=(63, 63))
         layer_record(c4["name"] + "_b64", c4["ops"], c4["bytes"], wall, dev, tm,
@@ -390,7 +404,8 @@ def main():
         if not ok:
             failures.append("cfg3 chain")
         layers.append({"layer": "cfg3_mobilenet_v1_0.5_128x128_b256 (whole chain)", "ms": round(dev, 5),
-                       "wall_ms": round(wall, 5), "timing": tm["device_us_per_step"], "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
+                       "wall_ms": round(wall, 5), "timing": tm["device_us_per_step"],
+                       "shader_mhz_behind_region": tm["shader_mhz_behind_region"], "gops": round(net["ops"] / (dev * 1e-3) / 1e9, 1),
                        "launches": runner.launches if hasattr(runner, "launches") else None,
                        "images_per_s": round(256 / (wall * 1e-3), 1),
                        "mfma_frac": round(net["ops"] / (dev * 1e-3) / PEAK_INT8_OPS, 4),

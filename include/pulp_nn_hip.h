@@ -39,6 +39,13 @@ void *pulp_nn_hip_get_stream(void);
 /* Wait for everything queued on the current stream.  Returns a status code. */
 int pulp_nn_hip_sync(void);
 
+/* Measurement aid (no counterpart in the reference): queues a one-wave kernel on the current stream that runs for
+ * 20 us and writes two 64-bit counts to device memory: out[0] = ticks of the 100 MHz wall clock, out[1] = cycles of the
+ * shader clock over the same interval (shader MHz = 100 * out[1] / out[0]).  Queued behind a run of layer calls it
+ * tells at which clock the GPU was left by them: the MFMA-bound layers run below the 2.4 GHz maximum under the
+ * power limit.  out: 16 bytes of device memory, 8-byte aligned. */
+void pulp_nn_hip_clock_probe(long long *out);
+
 /* Status of the most recent failing layer call on this thread since the last
  * pulp_nn_hip_clear_error(), or PULP_NN_HIP_OK.  A layer call that fails
  * validation queues no work. */

@@ -86,6 +86,8 @@ class PulpNN:
         L.pulp_nn_hip_set_stream.argtypes = [_PTR]
         L.pulp_nn_hip_get_stream.restype = _PTR
         L.pulp_nn_hip_sync.restype = _INT
+        L.pulp_nn_hip_clock_probe.argtypes = [_PTR]
+        L.pulp_nn_hip_clock_probe.restype = None
         L.pulp_nn_hip_last_error.restype = _INT
         L.pulp_nn_hip_last_error_string.restype = C.c_char_p
         L.pulp_nn_hip_bn_bits.restype = _INT
@@ -128,6 +130,10 @@ class PulpNN:
         rc = self._lib.pulp_nn_hip_sync()
         if rc:
             self._raise()
+
+    def clock_probe(self, out):
+        """Queues the 20 us clock probe; out: device tensor of two int64 (wall-clock ticks at 100 MHz, shader cycles)."""
+        self._call("pulp_nn_hip_clock_probe", _ptr(out))
 
     def last_error(self):
         return int(self._lib.pulp_nn_hip_last_error())

@@ -11,11 +11,15 @@
 // (102.8 MB in; 102.8 MB and 25.7 MB out) and the pointwise layer of config 1 (51.4 MB in, 25.7 MB out).
 // Four buffer pairs are used in turn (822 MB for the largest case: more than the 256 MB of last-level cache), one
 // event pair brackets 100 launches, the figure printed is the median of 8 such regions after 2 discarded ones.
+// Last, the approach to the settled rate from a cold start: region by region, with the shader clock read by a
+// one-wave probe kernel behind every region (a memory-bound kernel's time should not follow the shader clock; this
+// shows whether the slower first milliseconds of a run do).
 //
 // Build: hipcc --offload-arch=gfx950 -O3 -std=c++17 hbm_ceiling.hip -o hbm_ceiling   (python -m pulp_nn_amd.build does it)
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <unistd.h>
 #include <algorithm>
 #include <vector>
 
@@ -70,6 +74,19 @@ __global__ __launch_bounds__(256) void write_kernel(v4i *out, size_t n16, int pe
   for (int i = 0; i < per; i++) {
     const size_t idx = base + (size_t)i * 256;
     if (idx < n16) out[idx] = v4i{(int)idx, 1, 2, 3};
+  }
+}
+
+// shader clock right now: cycles of the shader counter per tick of the 100 MHz wall clock, over 20 us of one wave
+__global__ void clock_probe_kernel(long long *out)
+{
+  const long long t0 = wall_clock64(), c0 = __builtin_readcyclecounter();
+  long long t1 = t0;
+  while (t1 - t0 < 2000) t1 = wall_clock64();
+  const long long c1 = __builtin_readcyclecounter();
+  if (threadIdx.x == 0) {
+    out[0] = t1 - t0;
+    out[1] = c1 - c0;
   }
 }
 
@@ -128,6 +145,33 @@ int main()
     }
     if (c.in == c.out)
       timeit("hipMemcpyAsync device to device", 2.0 * c.in, [&](int i) { CK(hipMemcpyAsync(dout[i], din[i], c.in, hipMemcpyDeviceToDevice, 0)); });
+  }
+  // The approach to the settled rate: the pointwise layer's copy, 40 regions of 100 launches back to back from a cold
+  // start (the GPU idle for 100 ms before), with the shader clock read by a one-wave probe kernel behind every region.
+  {
+    const Case &c = cases[2];
+    const size_t n_in = c.in / 16, n_out = c.out / 16;
+    const int grid = (int)((n_in + 255) / 256);
+    long long *dprobe, hprobe[2];
+    CK(hipMalloc(&dprobe, 16));
+    CK(hipDeviceSynchronize());
+    usleep(100000);
+    printf("approach to the settled rate, %s copy (non-temporal, 1 x 4 KB per workgroup): us per launch (shader MHz behind the region)\n ", c.name);
+    double t_ms = 0;
+    for (int r = 0; r < 40; r++) {
+      CK(hipEventRecord(e0, 0));
+      for (int q = 0; q < 100; q++) hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(256), 0, 0, din[q % NBUF], dout[q % NBUF], n_in, n_out, 1);
+      CK(hipEventRecord(e1, 0));
+      hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, 0, dprobe);
+      CK(hipDeviceSynchronize());
+      float ms;
+      CK(hipEventElapsedTime(&ms, e0, e1));
+      CK(hipMemcpy(hprobe, dprobe, 16, hipMemcpyDeviceToHost));
+      t_ms += ms;
+      printf(" %.1f (%.0f)", ms * 10.f, hprobe[0] ? 100.0 * hprobe[1] / hprobe[0] : 0.0);
+      if (r % 10 == 9) printf("   [%.1f ms]\n ", t_ms);
+    }
+    printf("\n");
   }
   CK(hipGetLastError());
   return 0;

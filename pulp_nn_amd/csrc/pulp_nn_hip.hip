@@ -881,6 +881,20 @@ CalibGeom calib_conv_geom(const unsigned char *in, const signed char *bias, cons
 
 // ---- added entry points -----------------------------------------------------------
 
+// Shader clock right now: cycles of the shader counter against ticks of the 100 MHz wall clock, over 20 us of one
+// wave (pulp_nn_hip_clock_probe).
+__global__ void clock_probe_kernel(long long *out)
+{
+  const long long t0 = wall_clock64(), c0 = __builtin_readcyclecounter();
+  long long t1 = t0;
+  while (t1 - t0 < 2000) t1 = wall_clock64();
+  const long long c1 = __builtin_readcyclecounter();
+  if (threadIdx.x == 0) {
+    out[0] = t1 - t0;
+    out[1] = c1 - c0;
+  }
+}
+
 extern "C" {
 
 void pulp_nn_hip_set_batch(unsigned n_images)
@@ -900,6 +914,13 @@ int pulp_nn_hip_sync(void)
     return PULP_NN_HIP_ERR_RUNTIME;
   }
   return PULP_NN_HIP_OK;
+}
+
+void pulp_nn_hip_clock_probe(long long *out)
+{
+  REQUIRE(out && aligned(out, 8), PULP_NN_HIP_ERR_ARGUMENT, "null or misaligned pointer");
+  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, g_stream, out);
+  check_launch(__func__);
 }
 
 int pulp_nn_hip_last_error(void) { return g_err; }

@@ -379,3 +379,20 @@ def test_rejected_calls_report_an_error_and_write_nothing():
     L.sync()
     assert int(out.min()) == 0xA5
     assert L.last_error() == 0
+
+
+@pytest.mark.parametrize("bn_bits", [32, 64])
+def test_clock_probe_reads_a_plausible_shader_clock(bn_bits):
+    """pulp_nn_hip_clock_probe: 20 us of the 100 MHz wall clock and a shader clock between 0.3 and 3 GHz; a null
+    pointer is rejected."""
+    import torch
+    from pulp_nn_amd import PulpNNError
+    L = nn(bn_bits)
+    out = torch.zeros(2, dtype=torch.int64, device="cuda")
+    L.clock_probe(out)
+    L.sync()
+    ticks, cycles = (int(v) for v in out.cpu())
+    assert 2000 <= ticks < 20000, ticks
+    assert 300 <= 100.0 * cycles / ticks <= 3000, (ticks, cycles)
+    with pytest.raises(PulpNNError):
+        L.clock_probe(None)
