@@ -47,7 +47,7 @@ TRACE_FILE = os.path.join(ROOT, "profiles", "bench_all_layers_kernel_trace.txt")
 # regenerated shows up there.
 KERNELS = {
     "cfg1_pointwise": "pw_stream_kernel<4, 2, 4, 1, true, 1, 16>",
-    "cfg0_conv": "igemm_kernel<2, 2, 2, 3, 0, 4, 5>",
+    "cfg0_conv": "igemm_kernel<2, 4, 2, 3, 0, 2, 5>",
     "cfg2_dw_s1": "dw3x3_lin_kernel<1, 1, 0, true, true>",
     "cfg2_dw_s2": "dw3x3_stream_kernel<2, 1, 0>",
     "cfg4_conv": "igemm_patch_kernel<0, 0>",
